@@ -1,0 +1,169 @@
+/*
+ * C ABI of libiris_hip.so: hand-written gfx950 (MI355X) kernels for the rank-local compute of the
+ * fused GEMM+collective operators of the Iris Python package.
+ *
+ * The reference package has no native interface: each operator launches a Triton kernel through
+ * `iris_launch(kernel_fn, grid, *args, ...)` (iris/host/tracing/kernel_artifacts.py:54-83).  Every
+ * entry point below takes exactly the arguments of one such launch, in the same order and with the
+ * same meaning, followed by a short tail of values the Triton launch gets implicitly (element types,
+ * the HIP stream) or that this library adds (scales for fp8 inputs, a bound on flag spinning).
+ *
+ * Conventions
+ *   - All data pointers are device pointers.  Strides are in elements, as torch reports them.
+ *   - `context_tensor` is the int64 device array built by Iris._build_device_context
+ *     (iris/host/iris.py:916-958): [cur_rank, world_size, heap_base_0 .. heap_base_{W-1}, ...].
+ *     A pointer p inside slot `cur_rank` names, in slot r, the address
+ *     heap_base_r + (p - heap_base_cur_rank)   (iris/mem/triton/context.py:16-27).
+ *   - Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
+ *   - Return value: 0 on success, otherwise a hipError_t value.  Argument errors return
+ *     hipErrorInvalidValue (1); iris_hip_last_error() then describes the problem.
+ *   - The library allocates no device memory and keeps no state between calls.
+ */
+#ifndef IRIS_HIP_H
+#define IRIS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types (in_dtype / out_dtype / bias_dtype arguments). */
+enum {
+  IRIS_HIP_BF16 = 0,
+  IRIS_HIP_FP16 = 1,
+  IRIS_HIP_FP32 = 2,
+  IRIS_HIP_FP8_E4M3 = 3 /* OCP e4m3fn, inputs only; products are multiplied by `scale` */
+};
+
+/* All-reduce variants (the strings of FusedConfig.all_reduce_variant, iris/ops/config.py:62). */
+enum {
+  IRIS_HIP_VARIANT_ONE_SHOT = 2, /* iris/mem/triton/context.py:733-764 */
+  IRIS_HIP_VARIANT_TWO_SHOT = 3  /* iris/mem/triton/context.py:801-839 */
+};
+
+/* How the slot sum is carried (acc_mode). */
+enum {
+  IRIS_HIP_ACC_FP32 = 0,     /* fp32 running sum, one final cast */
+  IRIS_HIP_ACC_REFERENCE = 1 /* the reference rule: fp32 only for fp16 data, else the data type
+                                (bf16 sums are re-rounded after every add; context.py:752) */
+};
+
+/* Which A rows/columns come from which slot in iris_hip_all_gather_matmul (gather_dim). */
+enum {
+  IRIS_HIP_GATHER_K = 1, /* reference layout: slot r holds A[:, r*K_local:(r+1)*K_local] */
+  IRIS_HIP_GATHER_M = 2  /* slot r holds A[r*M_local:(r+1)*M_local, :]                    */
+};
+
+/* Kernel selection (path). */
+enum {
+  IRIS_HIP_PATH_AUTO = 0,   /* MFMA kernel when the operands qualify, else the generic kernel */
+  IRIS_HIP_PATH_MFMA = 1,   /* MFMA kernel or hipErrorInvalidValue */
+  IRIS_HIP_PATH_GENERIC = 2 /* generic kernel */
+};
+
+/* Bits set in *status by a kernel. */
+enum {
+  IRIS_HIP_STATUS_SPIN_TIMEOUT = 1 /* a peer flag did not become 1 within spin_limit polls */
+};
+
+/*
+ * Fused C = all_reduce(A @ B), rank-local part.
+ * Replaces the launch of _fused_matmul_all_reduce_kernel
+ * (iris/ops/matmul_all_reduce.py:334-362; kernel :25-145) for VARIANT one_shot / two_shot.
+ *
+ * Per flag tile t = pid_m * cdiv(N, block_size_n) + pid_n of block_size_m x block_size_n elements:
+ *   aux[tile]   = cast(A @ B)              (own slot)
+ *   locks[t]    = 1                        (own slot, after the aux stores are visible)
+ *   one_shot:   C[tile] = cast(own + sum_{r != cur_rank, ascending} aux@r[tile]) after locks@r[t] == 1
+ *   two_shot:   the same, only if t % world_size == cur_rank, and the result is also stored to
+ *               C@r[tile] for every other slot r.
+ * aux is addressed with C's strides, as the reference does (matmul_all_reduce.py:128).
+ *
+ * block_size_k is accepted for signature parity and does not change any result.
+ * scale multiplies the fp32 product before the cast (use scale_a*scale_b for fp8, 1.0f otherwise).
+ * spin_limit <= 0 spins without bound like the reference; > 0 gives up after that many polls of one
+ * flag and ORs IRIS_HIP_STATUS_SPIN_TIMEOUT into *status (status may be NULL).
+ */
+int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
+                               int64_t M, int64_t N, int64_t K,
+                               int64_t stride_am, int64_t stride_ak,
+                               int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm, int64_t stride_cn,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t variant,
+                               int32_t in_dtype, int32_t out_dtype, float scale, int32_t acc_mode,
+                               int64_t spin_limit, int32_t* status, int32_t path, void* stream);
+
+/*
+ * Fused C = reduce_scatter(A @ B), rank-local part.
+ * Replaces the launch of _fused_matmul_reduce_scatter_kernel
+ * (iris/ops/matmul_reduce_scatter.py:261-288; kernel :25-118; DeviceContext.reduce_scatter
+ * iris/mem/triton/context.py:953-997).
+ *
+ * aux and locks are written for every tile as above.  Flag tile t is owned by
+ * min(t / (tiles / world_size), world_size - 1); an owned tile is summed over the slots and stored to
+ * C in slot cur_rank at the tile's global coordinates.
+ *
+ * Two switches that the reference does not have serve a single GPU standing in for all W ranks:
+ *   all_owners != 0: the launch reduces every tile and stores tile t into C of slot owner(t).
+ *   sum_peers  == 0: peers contribute nothing (their flags are not read, their aux not loaded).
+ * The reference behaviour is all_owners = 0, sum_peers = 1.
+ */
+int iris_hip_matmul_reduce_scatter(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
+                                   int64_t M, int64_t N, int64_t K,
+                                   int64_t stride_am, int64_t stride_ak,
+                                   int64_t stride_bk, int64_t stride_bn,
+                                   int64_t stride_cm, int64_t stride_cn,
+                                   const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                                   int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                                   int32_t all_owners, int32_t sum_peers,
+                                   int32_t in_dtype, int32_t out_dtype, float scale, int32_t acc_mode,
+                                   int64_t spin_limit, int32_t* status, int32_t path, void* stream);
+
+/*
+ * Fused C = all_gather(A_sharded) @ B (+ bias[:, None]), rank-local part (pull pattern).
+ * Replaces the launch of _fused_all_gather_matmul_kernel
+ * (iris/ops/all_gather_matmul.py:266-300; kernel :26-159; DeviceContext.gather
+ * iris/mem/triton/context.py:866-888).
+ *
+ * A_sharded points at the shard in slot cur_rank; the shard of slot r sits at the same heap offset.
+ * gather_dim = IRIS_HIP_GATHER_K: A_sharded is M x K_local, K == world_size * K_local, and the
+ *   reduction runs over slot 0's columns, then slot 1's, ... (all_gather_matmul.py:94-122).
+ * gather_dim = IRIS_HIP_GATHER_M: A_sharded is (M / world_size) x K; output row m uses slot
+ *   m / (M / world_size).  K_local must equal K.
+ * bias (may be NULL) is a per-row vector of M elements of type bias_dtype, added in fp32 before the
+ * cast (all_gather_matmul.py:147-150).
+ */
+int iris_hip_all_gather_matmul(const void* A_sharded, const void* B, void* C, const void* bias,
+                               int64_t M, int64_t N, int64_t K, int64_t K_local,
+                               int64_t stride_am, int64_t stride_ak,
+                               int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm, int64_t stride_cn, int64_t stride_bias,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t gather_dim,
+                               int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype, float scale,
+                               int32_t path, void* stream);
+
+/*
+ * Device facts used by the host layer (reference: get_cu_count / get_num_xcc,
+ * iris/host/platform/hip.py:138,218).  Any output pointer may be NULL.
+ */
+int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_t* lds_bytes_per_block);
+
+/* Text of the last argument error reported on the calling thread ("" if none). */
+const char* iris_hip_last_error(void);
+
+/* Name of the kernel configuration the last successful launch on the calling thread used. */
+const char* iris_hip_last_kernel(void);
+
+/* ABI version of this header. */
+int iris_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IRIS_HIP_H */

@@ -1,0 +1,1160 @@
+// libiris_hip: gfx950 (MI355X) kernels for the rank-local compute of the fused GEMM+collective
+// operators, and the C ABI declared in include/iris_hip.h.
+//
+// Two kernels implement every operator:
+//
+//  * fused_mfma_kernel  - persistent tiled GEMM on the 32x32 MFMA blocks of CDNA4.  Operand tiles
+//    travel HBM -> LDS with 16-byte direct-to-LDS buffer loads into a ring of STAGES buffers
+//    (prefetch distance STAGES-1, one workgroup barrier per K step); the K-contiguous operand is
+//    read back with 16-byte LDS reads, the N-contiguous one with LDS transpose reads.  Each of the
+//    four waves owns a (BM/2)x(BN/2) block of fp32 accumulators.  Requires 16-byte aligned,
+//    unit-stride rows (see mfma_eligible()).
+//  * fused_generic_kernel - a plain 64x64 LDS-tiled FMA kernel for everything else (fp32 data,
+//    odd strides, sizes that are not multiples of 8 elements).
+//
+// Both end in the same epilogue protocol, which follows the reference kernels
+// (iris/ops/matmul_all_reduce.py:111-144, iris/ops/matmul_reduce_scatter.py:98-118,
+//  iris/mem/triton/context.py:733-764, 801-839, 953-997):
+//    1. cast the fp32 tile to the output type and store it to aux in the own slot,
+//    2. make those stores visible, then raise the flag of every finished flag tile,
+//    3. for the flag tiles this rank reduces: wait for the peers' flags, add the peers' aux tiles
+//       in ascending rank order, cast once, store to C (own slot; two-shot: every slot).
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "iris_hip.h"
+#include "layout.h"
+
+using namespace iris_layout;
+
+#define LDS_AS __attribute__((address_space(3)))
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+typedef __attribute__((ext_vector_type(4))) short i16x4_t;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+
+enum { EPI_STORE = 0, EPI_ONE_SHOT = 1, EPI_TWO_SHOT = 2, EPI_REDUCE_SCATTER = 3 };
+enum { GATHER_NONE = 0, GATHER_K = 1, GATHER_M = 2 };
+
+struct FusedParams {
+  const char* A;
+  const char* B;
+  char* C;
+  char* aux;
+  int* locks;
+  const char* bias;
+  int M, N, K;
+  int K_local;  // K extent held by one source slot (== K unless gathered along K)
+  int M_local;  // rows held by one source slot when gathered along M
+  int gather;
+  long long s_am, s_ak, s_bk, s_bn, s_cm, s_cn, s_bias;  // element strides
+  const long long* heap_bases;
+  int rank, world;
+  int flag_bm, flag_bn;
+  int epi;
+  int acc_mode;
+  int all_owners;
+  int sum_peers;
+  int bias_dtype;
+  float scale;
+  long long spin_limit;
+  int* status;
+  int tiles_m, tiles_n, group_m, num_xcd;
+};
+
+// ------------------------------------------------------------------------------------------------
+// Small device helpers
+// ------------------------------------------------------------------------------------------------
+
+// Address of `p` (a pointer into slot `from`) in slot `to`.
+__device__ __forceinline__ char* slot_ptr(const long long* heap_bases, const void* p, int from, int to) {
+  unsigned long long off = (unsigned long long)p - (unsigned long long)heap_bases[from];
+  return (char*)((unsigned long long)heap_bases[to] + off);
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(unsigned short b) { return __uint_as_float(((unsigned)b) << 16); }
+
+__device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
+  __bf16 h = (__bf16)f;  // round to nearest even; v_cvt_pk_bf16_f32 on gfx950
+  return __builtin_bit_cast(unsigned short, h);
+}
+__device__ __forceinline__ unsigned short float_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return __builtin_bit_cast(unsigned short, h);
+}
+__device__ __forceinline__ float f16_bits_to_float(unsigned short b) {
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+
+// Output element kinds of the 16-bit epilogue.
+struct OutBF16 {
+  static __device__ __forceinline__ float to_float(unsigned short b) { return bf16_bits_to_float(b); }
+  static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_bf16_bits(f); }
+  static constexpr bool kFp32SumInReference = false;
+};
+struct OutF16 {
+  static __device__ __forceinline__ float to_float(unsigned short b) { return f16_bits_to_float(b); }
+  static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_f16_bits(f); }
+  static constexpr bool kFp32SumInReference = true;
+};
+
+__device__ __forceinline__ float load_scalar_as_float(const char* base, long long idx, int dtype) {
+  if (dtype == IRIS_HIP_FP32) return ((const float*)base)[idx];
+  unsigned short b = ((const unsigned short*)base)[idx];
+  return dtype == IRIS_HIP_BF16 ? bf16_bits_to_float(b) : f16_bits_to_float(b);
+}
+
+__device__ __forceinline__ int owner_of(int epi, int t, int total, int world, int rank) {
+  if (epi == EPI_TWO_SHOT) return owner_interleaved(t, world);
+  if (epi == EPI_REDUCE_SCATTER) return owner_contiguous(t, total, world);
+  return rank;
+}
+
+// Raise the flags of the flag tiles covered by the macro tile at (m0, n0) of KM x KN elements.
+// Must be called by every thread of the workgroup after a release fence and a workgroup barrier
+// that follow the workgroup's aux stores.
+template <int KM, int KN, int NT>
+__device__ __forceinline__ void raise_flags(const FusedParams& p, int m0, int n0, int tid) {
+  const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
+  const int ftn = cdiv(p.N, p.flag_bn);
+  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
+  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
+  const int nfn = fn_hi - fn_lo + 1;
+  const int nft = (fm_hi - fm_lo + 1) * nfn;
+  for (int i = tid; i < nft; i += NT) {
+    const int fm = fm_lo + i / nfn, fn = fn_lo + i % nfn;
+    int* flag = p.locks + (fm * ftn + fn);
+    const int needed = macro_tiles_over_flag_tile(fm, fn, p.flag_bm, p.flag_bn, KM, KN, p.M, p.N);
+    bool last = true;
+    if (needed > 1) {
+      // Arrivals are counted in steps of 2 so that the flag never reads 1 before the last one.
+      int old = __hip_atomic_fetch_add(flag, 2, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
+      last = ((old >> 1) + 1) == needed;
+    }
+    if (last) __hip_atomic_exchange(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// Wait until the peers' flags of every flag tile this workgroup reduces are 1.
+template <int KM, int KN, int NT>
+__device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, int n0, int tid) {
+  const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
+  const int ftn = cdiv(p.N, p.flag_bn);
+  const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
+  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
+  const int nfn = fn_hi - fn_lo + 1;
+  const int nft = (fm_hi - fm_lo + 1) * nfn;
+  const int items = nft * p.world;
+  for (int i = tid; i < items; i += NT) {
+    const int r = i % p.world;
+    const int f = i / p.world;
+    if (r == p.rank) continue;
+    const int t = (fm_lo + f / nfn) * ftn + fn_lo + f % nfn;
+    if (!p.all_owners && owner_of(p.epi, t, ftotal, p.world, p.rank) != p.rank) continue;
+    const int* flag = (const int*)slot_ptr(p.heap_bases, p.locks + t, p.rank, r);
+    long long polls = 0;
+    while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != 1) {
+      if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
+        if (p.status) atomicOr(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// MFMA kernel configuration
+// ------------------------------------------------------------------------------------------------
+enum { IN_BF16 = 0, IN_F16 = 1, IN_FP8 = 2 };
+
+template <int IN_, int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool B_KCONTIG_>
+struct MfmaCfg {
+  static constexpr int IN = IN_;
+  static constexpr int ES = (IN_ == IN_FP8) ? 1 : 2;
+  static constexpr int CE = kChunkBytes / ES;           // elements per 16-byte chunk
+  static constexpr int KM = (IN_ == IN_FP8) ? 64 : 16;  // k per MFMA
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_;
+  static constexpr bool B_KCONTIG = B_KCONTIG_;
+  static constexpr int WM = WM_, WN = WN_, NW = WM_ * WN_, NT = 64 * NW;
+  static constexpr int TM = BM / WM, TN = BN / WN;  // per-wave block
+  static constexpr int MB = TM / 32, NB = TN / 32;  // 32x32 MFMA blocks per wave
+  static constexpr int KSLICES = BK / KM;
+  static constexpr int NFRAG = (IN_ == IN_FP8) ? 2 : 1;   // 16-byte pieces per operand fragment
+  static constexpr int RBA = BK * ES;                        // bytes per A tile row
+  static constexpr int RBB = B_KCONTIG ? BK * ES : BN * ES;  // bytes per B tile row
+  static constexpr int A_BYTES = BM * RBA;
+  static constexpr int B_BYTES = B_KCONTIG ? BN * RBB : BK * RBB;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LA = A_BYTES / kDmaBytes / NW;  // direct-to-LDS loads per thread per K step
+  static constexpr int LB = B_BYTES / kDmaBytes / NW;
+  static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+  // Epilogue staging: one 32-row slab of the wave's block, 16-bit elements, padded rows.
+  static constexpr int SROW = TN * 2 + 16;
+  static constexpr int STG_BYTES = 32 * SROW;
+  static constexpr int SMEM_BYTES = RING_BYTES > NW * STG_BYTES ? RING_BYTES : NW * STG_BYTES;
+  static_assert(A_BYTES % (kDmaBytes * NW) == 0 && B_BYTES % (kDmaBytes * NW) == 0, "tile/loader mismatch");
+  static_assert(BK % KM == 0 && TM % 32 == 0 && TN % 32 == 0, "tile/MFMA mismatch");
+  static_assert(STAGES >= 3, "the ring needs at least three slots");
+  static_assert((STAGES - 2) * (LA + LB) <= 63, "vmcnt field too small for this prefetch depth");
+};
+
+template <int IN>
+struct OutOf { using type = OutBF16; };
+template <>
+struct OutOf<IN_F16> { using type = OutF16; };
+
+// s_waitcnt vmcnt(n) with the other counters left unconstrained (gfx9 encoding).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+constexpr unsigned kInvalidOffset = 0x80000000u;
+
+// Buffer resource words for a raw buffer (stride 0) over [base, base + 2^31).  Bounds are enforced
+// per lane by the callers: an invalid lane presents offset 0x80000000, which is past num_records
+// and therefore loads zero.
+__device__ __forceinline__ i32x4_t make_rsrc_words(unsigned long long b) {
+  i32x4_t r;
+  r.x = __builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  r.y = __builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  r.z = 0x7FFFFFFF;
+  r.w = 0x00020000;
+  return r;
+}
+
+// One wave-wide 16-byte direct-to-LDS load: lane l deposits global bytes [voff + soff, +16) of the
+// buffer at LDS address lds_base + 16*l.  Written as inline assembly so that the compiler's
+// wait-count pass does not serialise LDS reads behind loads that target other ring slots; the
+// kernel orders them itself with wait_vmcnt() and workgroup barriers.
+__device__ __forceinline__ void dma16(i32x4_t rsrc, unsigned lds_base, unsigned voff, unsigned soff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
+// Read one accumulator register.  The "a" constraint keeps the MFMA results in the accumulation
+// registers until the epilogue consumes them, instead of copying all of them to VGPRs at once.
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  return (unsigned)(unsigned long long)(LDS_AS const char*)p;
+}
+
+template <class CFG>
+struct MfmaAcc {
+  f32x16_t v[CFG::MB][CFG::NB];
+};
+
+// Operand fragments of one k-slice for a wave's block.
+template <class CFG>
+struct Frags {
+  i32x4_t a[CFG::MB][CFG::NFRAG];
+  i32x4_t b[CFG::NB][CFG::NFRAG];
+};
+
+// One 32x32 MFMA with the operands in the order (B fragment, A fragment): the accumulator then
+// holds D[n][m], i.e. each lane owns 4 consecutive n for one m.
+template <int IN, int NF>
+__device__ __forceinline__ f32x16_t mfma_block(const i32x4_t (&a)[NF], const i32x4_t (&b)[NF], f32x16_t c) {
+  if constexpr (IN == IN_BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, b[0]),
+                                                   __builtin_bit_cast(bf16x8_t, a[0]), c, 0, 0, 0);
+  } else if constexpr (IN == IN_F16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, b[0]),
+                                                  __builtin_bit_cast(f16x8_t, a[0]), c, 0, 0, 0);
+  } else {
+    i32x8_t av, bv;
+    av.lo = a[0]; av.hi = a[1];
+    bv.lo = b[0]; bv.hi = b[1];
+    // cbsz = blgp = 0 selects e4m3 for both operands; scale bytes 0x7F are 2^0.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+}
+
+constexpr int kMaxCachedSlots = 8;  // heap bases kept in registers; larger worlds re-load them
+
+// ------------------------------------------------------------------------------------------------
+// MFMA kernel
+// ------------------------------------------------------------------------------------------------
+template <class CFG>
+__global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p) {
+  using Out = typename OutOf<CFG::IN>::type;
+  using ATile = RowTile<CFG::RBA>;
+  constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
+  constexpr int MB = CFG::MB, NB = CFG::NB, TM = CFG::TM, TN = CFG::TN, NW = CFG::NW, NT = CFG::NT;
+  constexpr int STAGES = CFG::STAGES, LA = CFG::LA, LB = CFG::LB, NFRAG = CFG::NFRAG, KS = CFG::KSLICES;
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / CFG::WN, wn = wave % CFG::WN;
+
+  // Heap bases of the first slots, read once (scalar loads) before the kernel stores anything.
+  unsigned long long hb[kMaxCachedSlots];
+#pragma unroll
+  for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (p.heap_bases && r < p.world) ? (unsigned long long)p.heap_bases[r] : 0ull;
+  const unsigned long long hb_own = p.heap_bases ? (unsigned long long)p.heap_bases[p.rank] : 0ull;
+  auto heap_base = [&](int r) -> unsigned long long {
+    unsigned long long v = 0;
+    if (r < kMaxCachedSlots) {
+#pragma unroll
+      for (int q = 0; q < kMaxCachedSlots; ++q) v = (r == q) ? hb[q] : v;
+    } else {
+      v = (unsigned long long)p.heap_bases[r];
+    }
+    return v;
+  };
+  // Address in slot r of own-slot address `own`.
+  auto in_slot = [&](unsigned long long own, int r) -> unsigned long long { return heap_base(r) + (own - hb_own); };
+
+  // ---- loader descriptors (tile independent) ---------------------------------------------------
+  // A: row tile [BM][RBA].
+  int la_row[LA], la_k[LA];
+  unsigned la_off[LA];
+#pragma unroll
+  for (int i = 0; i < LA; ++i) {
+    int row, c;
+    ATile::from_lds((wave + i * NW) * kDmaBytes + lane * kChunkBytes, row, c);
+    la_row[i] = row;
+    la_k[i] = c * CE;
+    la_off[i] = (unsigned)(row * p.s_am * ES + c * kChunkBytes);
+  }
+  // B: col tile [BK][BN*ES] (row-major B) or row tile [BN][RBA] (B given K-contiguous).
+  int lb_row[LB], lb_col[LB];  // col tile: (k row, n element); row tile: (n row, k element)
+  unsigned lb_off[LB];
+#pragma unroll
+  for (int i = 0; i < LB; ++i) {
+    int row, c;
+    const int off = (wave + i * NW) * kDmaBytes + lane * kChunkBytes;
+    if constexpr (CFG::B_KCONTIG) {
+      RowTile<CFG::RBB>::from_lds(off, row, c);
+      lb_off[i] = (unsigned)(row * p.s_bn * ES + c * kChunkBytes);
+    } else {
+      ColTile<CFG::RBB, ES>::from_lds(off, row, c);
+      lb_off[i] = (unsigned)(row * p.s_bk * ES + c * kChunkBytes);
+    }
+    lb_row[i] = row;
+    lb_col[i] = c * CE;
+  }
+
+  // ---- fragment read offsets (relative to the slot's A / B region) -------------------------------
+  int fa_off[KS][NFRAG];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+    for (int h = 0; h < NFRAG; ++h) {
+      const int c = (CFG::IN == IN_FP8) ? frag8_chunk(lane, kk, h) : frag16_chunk(lane, kk);
+      fa_off[kk][h] = ATile::lds_offset(wm * TM + frag16_row(lane), c);
+    }
+  // B operand: K-contiguous B reads exactly like A; row-major B uses transpose reads.
+  constexpr int NTR = (CFG::IN == IN_FP8) ? 1 : 2;  // distinct swizzles among the transpose reads
+  int fb_off[CFG::B_KCONTIG ? KS : NB][CFG::B_KCONTIG ? NFRAG : NTR];
+  if constexpr (CFG::B_KCONTIG) {
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+      for (int h = 0; h < NFRAG; ++h) {
+        const int c = (CFG::IN == IN_FP8) ? frag8_chunk(lane, kk, h) : frag16_chunk(lane, kk);
+        fb_off[kk][h] = RowTile<CFG::RBB>::lds_offset(wn * TN + frag16_row(lane), c);
+      }
+  } else {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int j = 0; j < NTR; ++j) {
+        int krow, n;
+        if constexpr (CFG::IN == IN_FP8) {
+          krow = tr8_krow(lane, 0, 0);
+          n = wn * TN + nb * 32 + tr8_ncol(lane);
+        } else {
+          krow = tr16_krow(lane, 0, j);
+          n = wn * TN + nb * 32 + tr16_ncol(lane);
+        }
+        fb_off[nb][j] = ColTile<CFG::RBB, ES>::lds_offset(krow, n / CE) + (n % CE) * ES;
+      }
+  }
+
+  // Read the fragments of k-slice kk of ring slot `slot`.
+  auto load_frags = [&](Frags<CFG>& f, int slot, int kk) {
+    const char* sa = smem + slot * CFG::STAGE_BYTES;
+    const char* sb = sa + CFG::A_BYTES;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      if constexpr (CFG::B_KCONTIG) {
+#pragma unroll
+        for (int h = 0; h < NFRAG; ++h)
+          f.b[nb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sb + fb_off[kk][h] + nb * 32 * CFG::RBB);
+      } else if constexpr (CFG::IN == IN_FP8) {
+        i32x2_t t[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          t[r] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (LDS_AS i32x2_t*)(LDS_AS char*)(sb + fb_off[nb][0] + (kk * 64 + 8 * r) * CFG::RBB));
+        f.b[nb][0] = (i32x4_t){t[0].x, t[0].y, t[1].x, t[1].y};
+        f.b[nb][NFRAG - 1] = (i32x4_t){t[2].x, t[2].y, t[3].x, t[3].y};
+      } else {
+        i16x4_t t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (LDS_AS i16x4_t*)(LDS_AS char*)(sb + fb_off[nb][0] + kk * 16 * CFG::RBB));
+        i16x4_t t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (LDS_AS i16x4_t*)(LDS_AS char*)(sb + fb_off[nb][NTR - 1] + kk * 16 * CFG::RBB));
+        i32x2_t u0 = __builtin_bit_cast(i32x2_t, t0), u1 = __builtin_bit_cast(i32x2_t, t1);
+        f.b[nb][0] = (i32x4_t){u0.x, u0.y, u1.x, u1.y};
+      }
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int h = 0; h < NFRAG; ++h)
+        f.a[mb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sa + fa_off[kk][h] + mb * 32 * CFG::RBA);
+  };
+
+  const int total_tiles = p.tiles_m * p.tiles_n;
+  const int nsrc = (p.gather == GATHER_K) ? p.world : 1;
+  const int klocal = (p.gather == GATHER_K) ? p.K_local : p.K;
+  const int nkb = cdiv(klocal, BK);
+  const int nsteps = nsrc * nkb;
+  char* const stg = smem + wave * CFG::STG_BYTES;
+  const unsigned smem_base = __builtin_amdgcn_readfirstlane(lds_address(smem));
+  const unsigned long long a_own = (unsigned long long)p.A;
+
+  for (int it = 0;; ++it) {
+    const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
+    if (tidx < 0) break;
+    int tm, tn;
+    grouped_tile(tidx, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- per-tile loader state ---------------------------------------------------------------
+    // Row validity is folded into the per-lane offsets once per tile.
+    unsigned a_voff[LA], b_voff[LB];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) a_voff[i] = (m0 + la_row[i] < p.M) ? la_off[i] : kInvalidOffset;
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+      if constexpr (CFG::B_KCONTIG)
+        b_voff[i] = (n0 + lb_row[i] < p.N) ? lb_off[i] : kInvalidOffset;
+      else
+        b_voff[i] = (n0 + lb_col[i] < p.N) ? lb_off[i] : kInvalidOffset;
+    }
+    // Byte offset of this tile's first A row inside the slot that holds it.
+    int a_slot = p.rank;
+    long long a_row0 = m0;
+    if (p.gather == GATHER_M) {
+      a_slot = m0 / p.M_local;
+      a_row0 = m0 - (long long)a_slot * p.M_local;
+    }
+    if (p.gather == GATHER_K) a_slot = 0;
+    const unsigned long long a_tile_off = (unsigned long long)(a_row0 * p.s_am * ES);
+    const i32x4_t rb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)n0 * (CFG::B_KCONTIG ? p.s_bn : 1) * ES);
+    i32x4_t ra = make_rsrc_words((p.gather == GATHER_NONE ? a_own : in_slot(a_own, a_slot)) + a_tile_off);
+
+    // Loader position: next K step to issue = (i_src, i_kb), i_step overall.
+    int i_step = 0, i_src = 0, i_kb = 0;
+
+    // Issue the direct-to-LDS loads of the next K step into ring slot `slot`.  Steps past the end
+    // load nothing (every lane is out of range and deposits zeros), which keeps the per-thread
+    // count of outstanding loads identical on every step.
+    auto issue = [&](int slot) {
+      const bool live = i_step < nsteps;
+      const int k0 = i_kb * BK;
+      const int klim = live ? klocal - k0 : 0;  // k elements of this step that exist
+      const unsigned sa = smem_base + slot * CFG::STAGE_BYTES + wave * kDmaBytes;
+      const unsigned sb = sa + CFG::A_BYTES;
+      const unsigned a_soff = (unsigned)(k0 * ES);
+      const long long kglob = (long long)i_src * klocal + k0;
+#pragma unroll
+      for (int i = 0; i < LA; ++i) {
+        const unsigned v = (la_k[i] < klim) ? a_voff[i] : kInvalidOffset;
+        dma16(ra, sa + i * NW * kDmaBytes, v, a_soff);
+      }
+      const unsigned b_soff = __builtin_amdgcn_readfirstlane(
+          CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
+#pragma unroll
+      for (int i = 0; i < LB; ++i) {
+        const int kpos = CFG::B_KCONTIG ? lb_col[i] : lb_row[i];
+        const unsigned v = (kpos < klim) ? b_voff[i] : kInvalidOffset;
+        dma16(rb, sb + i * NW * kDmaBytes, v, b_soff);
+      }
+      ++i_step;
+      if (++i_kb == nkb) {  // next source slot (gather along K only)
+        i_kb = 0;
+        ++i_src;
+        if (p.gather == GATHER_K && i_src < nsrc) ra = make_rsrc_words(in_slot(a_own, i_src) + a_tile_off);
+      }
+    };
+
+    MfmaAcc<CFG> acc;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc.v[mb][nb][i] = 0.f;
+
+    // ---- prologue: fill STAGES-1 ring slots, wait for the first ----------------------------------
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) issue(s);
+    wait_vmcnt<(STAGES - 2) * (LA + LB)>();
+    __builtin_amdgcn_s_barrier();
+    Frags<CFG> fr[2];
+    load_frags(fr[0], 0, 0);
+
+    // ---- main loop ----------------------------------------------------------------------------
+    // Invariant at the top of step s: the operands of step s are in LDS and visible to all waves,
+    // and the fragments of its first k-slice are in flight.  The step first makes sure step s+1
+    // has landed too, so that its first fragments can be fetched while step s still computes.
+    int slot = 0;
+    for (int s = 0; s < nsteps; ++s) {
+      // LDS is one coherent memory per CU, so a bare s_barrier (no fence, hence no forced wait for
+      // the fragment reads in flight) orders the operand ring between the waves.
+      wait_vmcnt<(STAGES - 3) * (LA + LB)>();  // this thread's loads of step s+1 have landed
+      __builtin_amdgcn_s_barrier();             // everyone's have; everyone is past step s-1
+      {
+        int pslot = slot + STAGES - 1;
+        if (pslot >= STAGES) pslot -= STAGES;
+        issue(pslot);                           // refill the slot step s-1 used
+      }
+      const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) {
+        if (kk + 1 < KS)
+          load_frags(fr[(kk + 1) & 1], slot, kk + 1);
+        else
+          load_frags(fr[(kk + 1) & 1], nslot, 0);
+        const Frags<CFG>& f = fr[kk & 1];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(f.a[mb], f.b[nb], acc.v[mb][nb]);
+      }
+      static_assert(KS % 2 == 0 || KS == 1, "fragment double buffer assumes an even slice count");
+      if constexpr (KS == 1) {
+        // With one slice per step the two buffers alternate across steps.
+        Frags<CFG> t = fr[0];
+        fr[0] = fr[1];
+        fr[1] = t;
+      }
+      slot = nslot;
+    }
+
+    // The ring is reused as epilogue staging: drain the (empty) loads still in flight and make
+    // sure every wave has finished reading operands.
+    wait_vmcnt<0>();
+    __syncthreads();
+
+    // ---- epilogue -------------------------------------------------------------------------------
+    const int wrow0 = m0 + wm * TM;  // first row / column of this wave's block
+    const int wcol0 = n0 + wn * TN;
+    constexpr int CPR = TN / 8;      // 16-byte chunks per staged row
+    constexpr int RPI = 64 / CPR;    // staged rows covered by one wave-wide access
+    constexpr int ITERS = 32 / RPI;
+    const int rd_row = lane / CPR, rd_chunk = lane % CPR;
+    const int ftn = cdiv(p.N, p.flag_bn);
+    const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+
+    // Write slab mb (32 rows of the wave's block) to the wave's staging area as 16-bit elements.
+    auto stage_slab = [&](int mb, const f32x16_t (&blk)[NB]) {
+      float badd = 0.f;
+      if (p.bias) {
+        const int gm = wrow0 + mb * 32 + acc_col(lane);
+        if (gm < p.M) badd = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          unsigned short h[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[e] = Out::from_float(acc_read(blk[nb][4 * q + e]) * p.scale + badd);
+          u32x2_t w;
+          w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
+          w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+          const int ncol = nb * 32 + acc_row(lane, 4 * q);
+          *(LDS_AS u32x2_t*)(LDS_AS char*)(stg + acc_col(lane) * CFG::SROW + ncol * 2) = w;
+        }
+      __builtin_amdgcn_wave_barrier();
+    };
+
+    // Phase 1: C (plain store) or aux (own slot).
+    char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      stage_slab(mb, acc.v[mb]);
+#pragma unroll
+      for (int i = 0; i < ITERS; ++i) {
+        const int r = i * RPI + rd_row;
+        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(stg + r * CFG::SROW + rd_chunk * 16);
+        const int gm = wrow0 + mb * 32 + r, gn = wcol0 + rd_chunk * 8;
+        if (gm < p.M && gn < p.N) *(u32x4_t*)(out1 + ((long long)gm * p.s_cm + gn) * 2) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+
+    if (p.epi != EPI_STORE) {
+      __atomic_thread_fence(__ATOMIC_RELEASE);  // system scope: the aux stores precede the flags
+      __syncthreads();
+      raise_flags<BM, BN, NT>(p, m0, n0, tid);
+      if (p.sum_peers && p.world > 1) {
+        wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
+        __syncthreads();
+      }
+
+      // Phase 2: reduce the flag tiles this rank is responsible for.
+      const bool ref_chain = (p.acc_mode == IRIS_HIP_ACC_REFERENCE) && !Out::kFp32SumInReference;
+      const unsigned long long aux_own = (unsigned long long)p.aux, c_own = (unsigned long long)p.C;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        stage_slab(mb, acc.v[mb]);
+#pragma unroll 2
+        for (int i = 0; i < ITERS; ++i) {
+          const int r = i * RPI + rd_row;
+          const u32x4_t own = *(const LDS_AS u32x4_t*)(LDS_AS char*)(stg + r * CFG::SROW + rd_chunk * 16);
+          const int gm = wrow0 + mb * 32 + r, gn = wcol0 + rd_chunk * 8;
+          if (!(gm < p.M && gn < p.N)) continue;
+          const int t = (gm / p.flag_bm) * ftn + gn / p.flag_bn;
+          const int owner = owner_of(p.epi, t, ftotal, p.world, p.rank);
+          if (!p.all_owners && owner != p.rank) continue;
+          const long long eoff = ((long long)gm * p.s_cm + gn) * 2;
+          float sum[8];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sum[2 * e] = Out::to_float((unsigned short)(own[e] & 0xFFFF));
+            sum[2 * e + 1] = Out::to_float((unsigned short)(own[e] >> 16));
+          }
+          if (p.sum_peers) {
+            for (int rb0 = 0; rb0 < p.world; rb0 += kMaxCachedSlots) {
+              u32x4_t pv[kMaxCachedSlots];
+#pragma unroll
+              for (int j = 0; j < kMaxCachedSlots; ++j) {
+                const int pr = rb0 + j;
+                if (pr < p.world && pr != p.rank) {
+                  const unsigned long long base = (rb0 == 0 ? hb[j] : (unsigned long long)p.heap_bases[pr]) + (aux_own - hb_own);
+                  pv[j] = *(const u32x4_t*)(base + eoff);
+                }
+              }
+#pragma unroll
+              for (int j = 0; j < kMaxCachedSlots; ++j) {
+                const int pr = rb0 + j;
+                if (pr < p.world && pr != p.rank) {
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) {
+                    sum[2 * e] += Out::to_float((unsigned short)(pv[j][e] & 0xFFFF));
+                    sum[2 * e + 1] += Out::to_float((unsigned short)(pv[j][e] >> 16));
+                  }
+                  if (ref_chain) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
+                  }
+                }
+              }
+            }
+          }
+          u32x4_t res;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
+          if (p.epi == EPI_TWO_SHOT) {
+            *(u32x4_t*)(c_own + eoff) = res;
+            for (int pr = 0; pr < p.world; ++pr)
+              if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff) = res;
+          } else {
+            const int dst = p.all_owners ? owner : p.rank;
+            *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff) = res;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
+    // Staging shares LDS with the operand ring of the next tile.
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Generic kernel: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMA.
+// ------------------------------------------------------------------------------------------------
+struct ElemBF16 {
+  static constexpr int size = 2;
+  static __device__ __forceinline__ float load(const char* p) { return bf16_bits_to_float(*(const unsigned short*)p); }
+  static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_bf16_bits(f); }
+  static __device__ __forceinline__ float round(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
+  static constexpr bool kFp32SumInReference = false;
+};
+struct ElemF16 {
+  static constexpr int size = 2;
+  static __device__ __forceinline__ float load(const char* p) { return f16_bits_to_float(*(const unsigned short*)p); }
+  static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_f16_bits(f); }
+  static __device__ __forceinline__ float round(float f) { return f16_bits_to_float(float_to_f16_bits(f)); }
+  static constexpr bool kFp32SumInReference = true;
+};
+struct ElemF32 {
+  static constexpr int size = 4;
+  static __device__ __forceinline__ float load(const char* p) { return *(const float*)p; }
+  static __device__ __forceinline__ void store(char* p, float f) { *(float*)p = f; }
+  static __device__ __forceinline__ float round(float f) { return f; }
+  static constexpr bool kFp32SumInReference = false;  // fp32 data sums in fp32 either way
+};
+struct ElemFP8 {
+  static constexpr int size = 1;
+  static __device__ __forceinline__ float load(const char* p) {
+    return __builtin_amdgcn_cvt_f32_fp8((int)*(const unsigned char*)p, 0);
+  }
+};
+
+constexpr int GT = 64;   // generic tile edge
+constexpr int GK = 16;   // generic k step
+
+template <class In, class Out>
+__global__ void __launch_bounds__(256) fused_generic_kernel(const FusedParams p) {
+  __shared__ float As[GK][GT + 1];
+  __shared__ float Bs[GK][GT + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int total_tiles = p.tiles_m * p.tiles_n;
+  const int ftn = cdiv(p.N, p.flag_bn);
+  const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+  const int nsrc = (p.gather == GATHER_K) ? p.world : 1;
+  const int klocal = (p.gather == GATHER_K) ? p.K_local : p.K;
+
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+    const int m0 = tm * GT, n0 = tn * GT;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+    for (int src = 0; src < nsrc; ++src) {
+      for (int k0 = 0; k0 < klocal; k0 += GK) {
+        // A tile: GT rows x GK k; thread loads 4 elements.
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int idx = tid + e * 256;  // 0..1023
+          const int r = idx / GK, kk = idx % GK;
+          const int gm = m0 + r, kl = k0 + kk;
+          float v = 0.f;
+          if (gm < p.M && kl < klocal) {
+            int slot = p.rank;
+            long long row = gm;
+            if (p.gather == GATHER_K) slot = src;
+            if (p.gather == GATHER_M) { slot = gm / p.M_local; row = gm - (long long)slot * p.M_local; }
+            const char* base = p.gather == GATHER_NONE ? p.A : slot_ptr(p.heap_bases, p.A, p.rank, slot);
+            v = In::load(base + (row * p.s_am + (long long)kl * p.s_ak) * In::size);
+          }
+          As[kk][r] = v;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int idx = tid + e * 256;
+          const int kk = idx / GT, c = idx % GT;
+          const int gn = n0 + c, kl = k0 + kk;
+          float v = 0.f;
+          if (gn < p.N && kl < klocal) {
+            const long long kg = (long long)src * klocal + kl;
+            v = In::load(p.B + (kg * p.s_bk + (long long)gn * p.s_bn) * In::size);
+          }
+          Bs[kk][c] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GK; ++kk) {
+          float a[4], b[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+      }
+    }
+
+    // Own tile, rounded to the output type.
+    float own[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int gm = m0 + ty * 4 + i;
+      float badd = 0.f;
+      if (p.bias && gm < p.M) badd = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) own[i][j] = Out::round(acc[i][j] * p.scale + badd);
+    }
+    char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int gm = m0 + ty * 4 + i, gn = n0 + tx * 4 + j;
+        if (gm < p.M && gn < p.N) Out::store(out1 + ((long long)gm * p.s_cm + (long long)gn * p.s_cn) * Out::size, own[i][j]);
+      }
+    if (p.epi == EPI_STORE) continue;
+
+    __atomic_thread_fence(__ATOMIC_RELEASE);
+    __syncthreads();
+    raise_flags<GT, GT, 256>(p, m0, n0, tid);
+    if (p.sum_peers && p.world > 1) {
+      wait_peer_flags<GT, GT, 256>(p, m0, n0, tid);
+      __syncthreads();
+    }
+    const bool ref_chain = (p.acc_mode == IRIS_HIP_ACC_REFERENCE) && !Out::kFp32SumInReference;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int gm = m0 + ty * 4 + i, gn = n0 + tx * 4 + j;
+        if (!(gm < p.M && gn < p.N)) continue;
+        const int t = (gm / p.flag_bm) * ftn + gn / p.flag_bn;
+        const int owner = owner_of(p.epi, t, ftotal, p.world, p.rank);
+        if (!p.all_owners && owner != p.rank) continue;
+        const long long eoff = ((long long)gm * p.s_cm + (long long)gn * p.s_cn) * Out::size;
+        float sum = own[i][j];
+        if (p.sum_peers)
+          for (int pr = 0; pr < p.world; ++pr) {
+            if (pr == p.rank) continue;
+            sum += Out::load(slot_ptr(p.heap_bases, p.aux, p.rank, pr) + eoff);
+            if (ref_chain) sum = Out::round(sum);
+          }
+        if (p.epi == EPI_TWO_SHOT) {
+          Out::store(p.C + eoff, sum);
+          for (int pr = 0; pr < p.world; ++pr)
+            if (pr != p.rank) Out::store(slot_ptr(p.heap_bases, p.C, p.rank, pr) + eoff, sum);
+        } else {
+          const int dst = p.all_owners ? owner : p.rank;
+          Out::store(slot_ptr(p.heap_bases, p.C, p.rank, dst) + eoff, sum);
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+thread_local char g_last_error[512] = "";
+thread_local char g_last_kernel[128] = "";
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return (int)hipErrorInvalidValue;
+}
+
+struct DeviceFacts {
+  int cu_count = 0;
+  int xcc_count = 0;
+  int lds_per_block = 0;
+  bool ok = false;
+};
+
+DeviceFacts g_facts[64];
+
+int facts_for(int device, DeviceFacts** out) {
+  if (device < 0 || device >= 64) return fail("device index %d out of range", device);
+  DeviceFacts& f = g_facts[device];
+  if (!f.ok) {
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return (int)e;
+    f.cu_count = prop.multiProcessorCount;
+    f.lds_per_block = (int)prop.sharedMemPerBlock;
+    // MI300/MI350-class parts expose 8 XCDs; smaller parts have one.
+    f.xcc_count = (f.cu_count >= 64 && f.cu_count % 8 == 0) ? 8 : 1;
+    f.ok = true;
+  }
+  *out = &f;
+  return 0;
+}
+
+int elem_size(int dtype) {
+  switch (dtype) {
+    case IRIS_HIP_BF16: case IRIS_HIP_FP16: return 2;
+    case IRIS_HIP_FP32: return 4;
+    case IRIS_HIP_FP8_E4M3: return 1;
+  }
+  return 0;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// Reasons (if any) the MFMA kernel cannot take these operands.
+const char* mfma_ineligible(const FusedParams& p, int in_dtype, int out_dtype, int bm, int bn) {
+  if (in_dtype == IRIS_HIP_FP32) return "fp32 inputs";
+  const int es = elem_size(in_dtype);
+  const int ce = 16 / es;
+  const int want_out = (in_dtype == IRIS_HIP_FP16) ? IRIS_HIP_FP16 : IRIS_HIP_BF16;
+  if (out_dtype != want_out) return "output type not paired with the input type";
+  if (p.s_ak != 1) return "A is not K-contiguous";
+  if (p.s_bn != 1 && p.s_bk != 1) return "B has no unit stride";
+  if (p.s_cn != 1) return "C is not N-contiguous";
+  if (!aligned16(p.A) || !aligned16(p.B) || !aligned16(p.C)) return "base pointers not 16-byte aligned";
+  if (p.aux && !aligned16(p.aux)) return "aux not 16-byte aligned";
+  if (p.K % ce || p.K_local % ce) return "K not a multiple of 16 bytes";
+  if ((p.s_am * es) % 16) return "A rows not 16-byte aligned";
+  if (p.s_bn == 1) {
+    if (p.N % ce) return "N not a multiple of 16 bytes of B";
+    if ((p.s_bk * es) % 16) return "B rows not 16-byte aligned";
+  } else {
+    if ((p.s_bn * es) % 16) return "B columns not 16-byte aligned";
+  }
+  if (p.N % 8 || p.s_cm % 8) return "C rows not 16-byte aligned";
+  if (p.flag_bn % 8) return "flag tile width not a multiple of 8";
+  // 32-bit buffer offsets: per-lane offset + per-step offset must stay below 2^31.
+  const long long a_span = (long long)bm * p.s_am * es + (long long)p.K * es;
+  const long long b_span = (p.s_bn == 1) ? (long long)p.K * p.s_bk * es + (long long)bn * es
+                                         : (long long)bn * p.s_bn * es + (long long)p.K * es;
+  if (a_span >= (1ll << 31) || b_span >= (1ll << 31)) return "operand too large for 32-bit tile offsets";
+  if (p.gather == GATHER_M && (p.M_local % bm)) return "M_local not a multiple of the tile height";
+  return nullptr;
+}
+
+template <class CFG>
+int launch_mfma(const FusedParams& p, int cu_count, hipStream_t stream, const char* name) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int total = p.tiles_m * p.tiles_n;
+  int grid = total < cu_count ? total : cu_count;
+  if (grid >= p.num_xcd) grid -= grid % p.num_xcd;  // keep the XCD mapping exact
+  if (grid < 1) grid = 1;
+  hipLaunchKernelGGL(fused_mfma_kernel<CFG>, dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
+  snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name);
+  return (int)hipGetLastError();
+}
+
+template <class In, class Out>
+int launch_generic(FusedParams p, int cu_count, hipStream_t stream, const char* name) {
+  p.tiles_m = cdiv(p.M, GT);
+  p.tiles_n = cdiv(p.N, GT);
+  const long long total = (long long)p.tiles_m * p.tiles_n;
+  const long long cap = (long long)cu_count * 8;
+  const int grid = (int)(total < cap ? total : cap);
+  hipLaunchKernelGGL((fused_generic_kernel<In, Out>), dim3(grid < 1 ? 1 : grid), dim3(256), 0, stream, p);
+  snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name);
+  return (int)hipGetLastError();
+}
+
+int dispatch_generic(const FusedParams& p, int in_dtype, int out_dtype, int cu, hipStream_t s) {
+#define GEN(I, O, name) return launch_generic<I, O>(p, cu, s, name)
+  if (in_dtype == IRIS_HIP_BF16 && out_dtype == IRIS_HIP_BF16) GEN(ElemBF16, ElemBF16, "generic_bf16");
+  if (in_dtype == IRIS_HIP_FP16 && out_dtype == IRIS_HIP_FP16) GEN(ElemF16, ElemF16, "generic_f16");
+  if (in_dtype == IRIS_HIP_FP32 && out_dtype == IRIS_HIP_FP32) GEN(ElemF32, ElemF32, "generic_f32");
+  if (in_dtype == IRIS_HIP_FP8_E4M3 && out_dtype == IRIS_HIP_BF16) GEN(ElemFP8, ElemBF16, "generic_fp8_bf16");
+  if (in_dtype == IRIS_HIP_FP8_E4M3 && out_dtype == IRIS_HIP_FP16) GEN(ElemFP8, ElemF16, "generic_fp8_f16");
+  if (in_dtype == IRIS_HIP_BF16 && out_dtype == IRIS_HIP_FP32) GEN(ElemBF16, ElemF32, "generic_bf16_f32");
+  if (in_dtype == IRIS_HIP_FP16 && out_dtype == IRIS_HIP_FP32) GEN(ElemF16, ElemF32, "generic_f16_f32");
+#undef GEN
+  return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
+}
+
+// Tile shapes of the MFMA kernel.  The large tile keeps 256 accumulator registers per lane busy;
+// the small one gives short problems enough workgroups to cover the 256 CUs.
+template <int IN, bool BKC>
+using BigTile = MfmaCfg<IN, 256, 256, (IN == IN_FP8 ? 64 : 32), 2, 4, 4, BKC>;
+template <int IN, bool BKC>
+using SmallTile = MfmaCfg<IN, 128, 128, (IN == IN_FP8 ? 64 : 32), 2, 2, 4, BKC>;
+
+template <int IN>
+int dispatch_mfma_in(FusedParams& p, bool big, bool bkc, int cu, hipStream_t s) {
+  const int bm = big ? 256 : 128, bn = bm;
+  p.tiles_m = cdiv(p.M, bm);
+  p.tiles_n = cdiv(p.N, bn);
+  // Group height: tile-rows walked together so that an XCD's span of tiles is close to square.
+  const int span = cdiv(p.tiles_m * p.tiles_n, p.num_xcd);
+  int g = 1;
+  while (g * g * 2 <= span && g * 2 <= p.tiles_m) g *= 2;
+  p.group_m = g;
+  static const char* names[3] = {"bf16", "f16", "fp8"};
+  char name[96];
+  snprintf(name, sizeof(name), "mfma_%s_%dx%dx%d_%s", names[IN], bm, bn, IN == IN_FP8 ? 64 : 32, bkc ? "nt" : "nn");
+  if (big) {
+    if (bkc) return launch_mfma<BigTile<IN, true>>(p, cu, s, name);
+    return launch_mfma<BigTile<IN, false>>(p, cu, s, name);
+  }
+  if (bkc) return launch_mfma<SmallTile<IN, true>>(p, cu, s, name);
+  return launch_mfma<SmallTile<IN, false>>(p, cu, s, name);
+}
+
+int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
+  g_last_error[0] = 0;
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("M, N, K must be positive (got %d, %d, %d)", p.M, p.N, p.K);
+  if (!p.A || !p.B || !p.C) return fail("A, B and C must not be NULL");
+  if (p.world < 1 || p.rank < 0 || p.rank >= p.world) return fail("bad rank/world_size %d/%d", p.rank, p.world);
+  if (p.epi != EPI_STORE) {
+    if (!p.aux || !p.locks) return fail("aux_buffer and locks must not be NULL");
+    if (p.flag_bm <= 0 || p.flag_bn <= 0) return fail("block sizes must be positive");
+  } else {
+    p.flag_bm = p.flag_bm > 0 ? p.flag_bm : 1;
+    p.flag_bn = p.flag_bn > 0 ? p.flag_bn : 1;
+  }
+  if ((p.world > 1 || p.gather != GATHER_NONE) && !p.heap_bases) return fail("context_tensor must not be NULL");
+  if (elem_size(in_dtype) == 0 || elem_size(out_dtype) == 0 || out_dtype == IRIS_HIP_FP8_E4M3)
+    return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
+
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return (int)e;
+  DeviceFacts* facts = nullptr;
+  int rc = facts_for(device, &facts);
+  if (rc) return rc;
+  p.num_xcd = facts->xcc_count;
+  hipStream_t s = (hipStream_t)stream;
+
+  // Tile choice: the 256x256 tile when it alone fills most of the machine, else 128x128.
+  const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
+  const bool big = big_tiles * 10 >= (long long)facts->cu_count * 8;
+  const int bm = big ? 256 : 128;
+  const char* why = mfma_ineligible(p, in_dtype, out_dtype, bm, bm);
+  if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
+  if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
+
+  const bool bkc = (p.s_bn != 1);
+  switch (in_dtype) {
+    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, big, bkc, facts->cu_count, s);
+    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, big, bkc, facts->cu_count, s);
+    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, big, bkc, facts->cu_count, s);
+  }
+  return fail("unsupported input type %d", in_dtype);
+}
+
+bool fits_int(int64_t v) { return v > 0 && v < (1ll << 31); }
+
+}  // namespace
+
+extern "C" {
+
+int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
+                               int64_t M, int64_t N, int64_t K,
+                               int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm, int64_t stride_cn,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t variant, int32_t in_dtype, int32_t out_dtype, float scale,
+                               int32_t acc_mode, int64_t spin_limit, int32_t* status, int32_t path,
+                               void* stream) {
+  (void)block_size_k;
+  if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
+  if (variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
+    return fail("variant %d is not one_shot (2) or two_shot (3)", variant);
+  FusedParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C; p.aux = (char*)aux_buffer; p.locks = locks;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.K_local = (int)K; p.gather = GATHER_NONE;
+  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
+  p.s_cm = stride_cm; p.s_cn = stride_cn;
+  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
+  p.rank = cur_rank; p.world = world_size;
+  p.flag_bm = block_size_m; p.flag_bn = block_size_n;
+  p.epi = variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
+  p.acc_mode = acc_mode; p.all_owners = 0; p.sum_peers = 1;
+  p.scale = scale; p.spin_limit = spin_limit; p.status = status;
+  return run_fused(p, in_dtype, out_dtype, path, stream);
+}
+
+int iris_hip_matmul_reduce_scatter(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
+                                   int64_t M, int64_t N, int64_t K,
+                                   int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                                   int64_t stride_cm, int64_t stride_cn,
+                                   const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                                   int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                                   int32_t all_owners, int32_t sum_peers,
+                                   int32_t in_dtype, int32_t out_dtype, float scale, int32_t acc_mode,
+                                   int64_t spin_limit, int32_t* status, int32_t path, void* stream) {
+  (void)block_size_k;
+  if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
+  FusedParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C; p.aux = (char*)aux_buffer; p.locks = locks;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.K_local = (int)K; p.gather = GATHER_NONE;
+  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
+  p.s_cm = stride_cm; p.s_cn = stride_cn;
+  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
+  p.rank = cur_rank; p.world = world_size;
+  p.flag_bm = block_size_m; p.flag_bn = block_size_n;
+  p.epi = EPI_REDUCE_SCATTER;
+  p.acc_mode = acc_mode; p.all_owners = all_owners ? 1 : 0; p.sum_peers = sum_peers ? 1 : 0;
+  p.scale = scale; p.spin_limit = spin_limit; p.status = status;
+  return run_fused(p, in_dtype, out_dtype, path, stream);
+}
+
+int iris_hip_all_gather_matmul(const void* A_sharded, const void* B, void* C, const void* bias,
+                               int64_t M, int64_t N, int64_t K, int64_t K_local,
+                               int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm, int64_t stride_cn, int64_t stride_bias,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t gather_dim, int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype,
+                               float scale, int32_t path, void* stream) {
+  (void)block_size_m; (void)block_size_n; (void)block_size_k;
+  if (!fits_int(M) || !fits_int(N) || !fits_int(K) || !fits_int(K_local))
+    return fail("M, N, K, K_local must be in [1, 2^31)");
+  FusedParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = (const char*)A_sharded; p.B = (const char*)B; p.C = (char*)C; p.bias = (const char*)bias;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  if (gather_dim == IRIS_HIP_GATHER_K) {
+    if (K != (int64_t)world_size * K_local)
+      return fail("K (%lld) must equal world_size (%d) * K_local (%lld)", (long long)K, world_size, (long long)K_local);
+    p.gather = GATHER_K; p.K_local = (int)K_local; p.M_local = (int)M;
+  } else if (gather_dim == IRIS_HIP_GATHER_M) {
+    if (K_local != K) return fail("gather along M needs K_local == K");
+    if (M % world_size) return fail("gather along M needs M divisible by world_size");
+    p.gather = GATHER_M; p.K_local = (int)K; p.M_local = (int)(M / world_size);
+  } else {
+    return fail("gather_dim %d is not 1 (K) or 2 (M)", gather_dim);
+  }
+  if (bias && elem_size(bias_dtype) < 2) return fail("unsupported bias type %d", bias_dtype);
+  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
+  p.s_cm = stride_cm; p.s_cn = stride_cn; p.s_bias = stride_bias; p.bias_dtype = bias_dtype;
+  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
+  p.rank = cur_rank; p.world = world_size;
+  p.epi = EPI_STORE; p.scale = scale;
+  return run_fused(p, in_dtype, out_dtype, path, stream);
+}
+
+int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_t* lds_bytes_per_block) {
+  g_last_error[0] = 0;
+  DeviceFacts* f = nullptr;
+  int rc = facts_for(device, &f);
+  if (rc) return rc;
+  if (cu_count) *cu_count = f->cu_count;
+  if (xcc_count) *xcc_count = f->xcc_count;
+  if (lds_bytes_per_block) *lds_bytes_per_block = f->lds_per_block;
+  return 0;
+}
+
+const char* iris_hip_last_error(void) { return g_last_error; }
+const char* iris_hip_last_kernel(void) { return g_last_kernel; }
+int iris_hip_abi_version(void) { return 1; }
+
+}  // extern "C"

@@ -1,0 +1,177 @@
+// Index math shared by the gfx950 GEMM kernels and the host-side layout simulator.
+//
+// Everything here is a pure function of small integers, usable from host and device code.
+// The kernels move operand tiles from HBM into LDS with 16-byte direct-to-LDS buffer loads
+// (one wave instruction deposits 64 lanes x 16 B = 1 KiB of contiguous LDS), read the
+// K-contiguous operand with 16-byte LDS reads and the N-contiguous operand with the gfx950
+// LDS transpose reads, and feed 32x32 MFMA blocks.  The functions below say, for every lane,
+// which global 16-byte chunk it fetches, where that chunk lives in LDS, and which LDS address
+// a lane presents when it assembles an MFMA operand.
+//
+// Conventions
+//   ES     element size in bytes (2 for bf16/fp16, 1 for fp8)
+//   chunk  16 bytes = CE elements (8 or 16)
+//   "row tile"   an operand tile stored as [rows][BK elements], K contiguous  (A, or B given as B^T)
+//   "col tile"   an operand tile stored as [BK rows (k)][BN elements], N contiguous (row-major B)
+#pragma once
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define IRIS_HD __host__ __device__ __forceinline__
+#else
+#define IRIS_HD inline
+#endif
+
+namespace iris_layout {
+
+constexpr int kChunkBytes = 16;
+constexpr int kWave = 64;
+constexpr int kDmaBytes = kWave * kChunkBytes;  // LDS bytes written by one wave-level load
+
+// ---------------------------------------------------------------------------------------------
+// Row tile: [rows][RB bytes], RB = BK*ES in {64, 128}.  16-byte chunks are XOR-swizzled so that
+// 16 lanes reading the same logical chunk of 16 consecutive rows touch 16 distinct 16-byte
+// bank groups (one full sweep of the 64 four-byte banks).
+// ---------------------------------------------------------------------------------------------
+template <int RB>
+struct RowTile {
+  static_assert(RB == 64 || RB == 128 || RB == 256, "row bytes must be 64, 128 or 256");
+  static constexpr int kChunksPerRow = RB / kChunkBytes;
+  static constexpr int kRowsPer256 = (256 / RB) > 0 ? (256 / RB) : 1;
+
+  IRIS_HD static int swizzle(int row) { return (row / kRowsPer256) % kChunksPerRow; }
+  // LDS byte offset of logical chunk c of a row.
+  IRIS_HD static int lds_offset(int row, int c) { return row * RB + ((c ^ swizzle(row)) * kChunkBytes); }
+  // Inverse used by the loader: LDS byte offset (multiple of 16) -> (row, logical chunk).
+  IRIS_HD static void from_lds(int off, int& row, int& c) {
+    row = off / RB;
+    c = ((off % RB) / kChunkBytes) ^ swizzle(row);
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Col tile: [BK rows][RB bytes], RB = BN*ES >= 256 (16-bit) or >= 128 (8-bit).  A 16-lane group
+// of a transpose read touches 4 k-rows x 32 B (16-bit) or 8 k-rows x 16 B (8-bit); rotating the
+// chunk index by the k-row keeps those on distinct banks.
+// ---------------------------------------------------------------------------------------------
+template <int RB, int ES>
+struct ColTile {
+  static_assert(ES == 1 || ES == 2, "element size must be 1 or 2 bytes");
+  static constexpr int kChunksPerRow = RB / kChunkBytes;
+  static constexpr int kSw = (ES == 2) ? 2 : 1;
+  static_assert(kChunksPerRow >= 8 * kSw, "tile row too short for the swizzle");
+
+  IRIS_HD static int swizzle(int krow) { return (krow % 8) * kSw; }
+  IRIS_HD static int lds_offset(int krow, int c) { return krow * RB + ((c ^ swizzle(krow)) * kChunkBytes); }
+  IRIS_HD static void from_lds(int off, int& krow, int& c) {
+    krow = off / RB;
+    c = ((off % RB) / kChunkBytes) ^ swizzle(krow);
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// MFMA 32x32 operand lanes.  For v_mfma_f32_32x32x16_{bf16,f16} lane l supplies, for row (or
+// column) l%32, the 8 k-values 8*(l/32)..+7 of the 16-wide k-slice; for the 8-bit 32x32x64 form
+// it supplies the 32 k-values 32*(l/32)..+31.  Only the pairing of A and B k-slots matters for
+// the product, so both operands simply use the same rule.
+// ---------------------------------------------------------------------------------------------
+
+// 16-bit, K-contiguous operand: one 16-byte read per 32x32x16 MFMA.
+//   row  = block_row0 + lane%32 ; chunk = kk*2 + lane/32        (kk = k-slice of 16 within the tile)
+IRIS_HD int frag16_row(int lane) { return lane % 32; }
+IRIS_HD int frag16_chunk(int lane, int kk) { return kk * 2 + lane / 32; }
+
+// 8-bit, K-contiguous operand: two 16-byte reads per 32x32x64 MFMA (h = 0,1).
+IRIS_HD int frag8_chunk(int lane, int kk, int h) { return kk * 4 + 2 * (lane / 32) + h; }
+
+// LDS transpose read, 16-bit (ds_read_b64_tr_b16).  Within each 16-lane group, lane p presents
+// the address of 4 consecutive n at k-row p/4, n = 4*(p%4); it receives, for n = p, the 4 k-rows.
+// For read j (0,1) of the k-slice kk, lane l of the wave addresses:
+IRIS_HD int tr16_krow(int lane, int kk, int j) {
+  int g = lane / 16, p = lane % 16;
+  return kk * 16 + 8 * (g / 2) + 4 * j + p / 4;
+}
+IRIS_HD int tr16_ncol(int lane) {  // first of 4 consecutive n, relative to the 32-wide block
+  int g = lane / 16, p = lane % 16;
+  return 16 * (g % 2) + 4 * (p % 4);
+}
+
+// LDS transpose read, 8-bit (ds_read_b64_tr_b8).  Lane p of a 16-lane group presents 8
+// consecutive n at k-row p/2, n = 8*(p%2); it receives, for n = p, the 8 k-rows.
+// For read r (0..3) of the 64-wide k-slice kk:
+IRIS_HD int tr8_krow(int lane, int kk, int r) {
+  int g = lane / 16, p = lane % 16;
+  return kk * 64 + 32 * (g / 2) + 8 * r + p / 2;
+}
+IRIS_HD int tr8_ncol(int lane) {
+  int g = lane / 16, p = lane % 16;
+  return 16 * (g % 2) + 8 * (p % 2);
+}
+
+// Accumulator of D = X * Y for the 32x32 MFMA: register i (0..15) of lane l holds
+//   D[row = 8*(i/4) + 4*(l/32) + i%4][col = l%32].
+// The kernels issue mfma(Bfrag, Afrag) so that D rows run along n and columns along m: every
+// lane then owns 4 consecutive n for one m, which packs into one 8-byte LDS write.
+IRIS_HD int acc_row(int lane, int i) { return 8 * (i / 4) + 4 * (lane / 32) + (i % 4); }
+IRIS_HD int acc_col(int lane) { return lane % 32; }
+
+// ---------------------------------------------------------------------------------------------
+// Tile order.  Workgroup b of a launch lands on XCD b % num_xcd (round-robin dispatch).  Tiles
+// are first put in a grouped order (group_m tile-rows at a time, walking down the group's
+// column before moving right) and each XCD is handed one contiguous span of that order, so the
+// tiles that share A row-panels and B column-panels meet in the same L2.
+// ---------------------------------------------------------------------------------------------
+IRIS_HD void grouped_tile(int idx, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
+  int per_group = group_m * tiles_n;
+  int g = idx / per_group;
+  int first_m = g * group_m;
+  int rows = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+  int r = idx - g * per_group;
+  tm = first_m + r % rows;
+  tn = r / rows;
+}
+
+// Position in the grouped order of the it-th tile processed by workgroup `wg` of `nwg`.
+// Returns -1 when that workgroup has no it-th tile.
+IRIS_HD int xcd_tile_index(int wg, int nwg, int it, int total, int num_xcd) {
+  if (nwg % num_xcd != 0 || nwg < num_xcd) {  // plain round-robin
+    long idx = (long)wg + (long)it * nwg;
+    return idx < total ? (int)idx : -1;
+  }
+  int xcd = wg % num_xcd;
+  int local = wg / num_xcd;
+  int wg_per_xcd = nwg / num_xcd;
+  int span = (total + num_xcd - 1) / num_xcd;
+  long in_span = (long)local + (long)it * wg_per_xcd;
+  if (in_span >= span) return -1;
+  long idx = (long)xcd * span + in_span;
+  return idx < total ? (int)idx : -1;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Flag tiles (the reference's BLOCK_SIZE_M x BLOCK_SIZE_N tiles) and their owners.
+// ---------------------------------------------------------------------------------------------
+IRIS_HD int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Owner of flag tile t under interleaved (two-shot all-reduce) distribution.
+IRIS_HD int owner_interleaved(int t, int world) { return t % world; }
+
+// Owner of flag tile t under contiguous (reduce-scatter) distribution: each rank takes
+// total/world tiles, the last rank also the remainder.
+IRIS_HD int owner_contiguous(int t, int total, int world) {
+  int per = total / world;
+  if (per == 0) return world - 1;
+  int o = t / per;
+  return o < world - 1 ? o : world - 1;
+}
+
+// How many kernel macro-tiles (KM x KN) overlap flag tile (fm, fn) of size (FM x FN) in an
+// M x N matrix.  A flag is raised by the last of them to finish.
+IRIS_HD int macro_tiles_over_flag_tile(int fm, int fn, int FM, int FN, int KM, int KN, int M, int N) {
+  int r0 = fm * FM, r1 = (fm + 1) * FM < M ? (fm + 1) * FM : M;
+  int c0 = fn * FN, c1 = (fn + 1) * FN < N ? (fn + 1) * FN : N;
+  int nm = (r1 - 1) / KM - r0 / KM + 1;
+  int nn = (c1 - 1) / KN - c0 / KN + 1;
+  return nm * nn;
+}
+
+}  // namespace iris_layout
