@@ -284,8 +284,9 @@ __device__ __forceinline__ f32x16_t mfma_block(const i32x4_t (&a)[NF], const i32
     i32x8_t av, bv;
     av.lo = a[0]; av.hi = a[1];
     bv.lo = b[0]; bv.hi = b[1];
-    // cbsz = blgp = 0 selects e4m3 for both operands; scale bytes 0x7F are 2^0.
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled
+    // instruction (v_mfma_f32_32x32x64_f8f6f4).
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 0, 0, 0, 0, 0, 0);
   }
 }
 
@@ -1014,8 +1015,8 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     if (!p.aux || !p.locks) return fail("aux_buffer and locks must not be NULL");
     if (p.flag_bm <= 0 || p.flag_bn <= 0) return fail("block sizes must be positive");
   } else {
-    p.flag_bm = p.flag_bm > 0 ? p.flag_bm : 1;
-    p.flag_bn = p.flag_bn > 0 ? p.flag_bn : 1;
+    p.flag_bm = 256;  // no flags on this path; any valid tile size
+    p.flag_bn = 64;
   }
   if ((p.world > 1 || p.gather != GATHER_NONE) && !p.heap_bases) return fail("context_tensor must not be NULL");
   if (elem_size(in_dtype) == 0 || elem_size(out_dtype) == 0 || out_dtype == IRIS_HIP_FP8_E4M3)

@@ -137,8 +137,6 @@ def matmul_all_reduce(
         raise NotImplementedError(
             f"all_reduce_variant {config.all_reduce_variant!r} has no HIP kernel; use 'one_shot' or 'two_shot'"
         )
-    require_gpu_tensors(shmem, A=A, B=B, C=C)
-
     needs_prepare = workspace is None or not workspace.matches(
         "matmul_all_reduce", (M, N, K), A.dtype, world_size, config.all_reduce_variant
     )
@@ -167,6 +165,7 @@ def matmul_all_reduce(
     elif scale_a is not None or scale_b is not None:
         raise ValueError("scale_a / scale_b only apply to float8 inputs")
 
+    require_gpu_tensors(shmem, A=A, B=B, C=C)
     iris_launch(
         "iris_hip_matmul_all_reduce",
         grid,

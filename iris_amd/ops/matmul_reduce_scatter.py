@@ -113,8 +113,6 @@ def matmul_reduce_scatter(
             raise ValueError(f"float8 inputs need a bfloat16/float16 output, got A:{A.dtype}, B:{B.dtype}, C:{C.dtype}")
     elif A.dtype != B.dtype or A.dtype != C.dtype:
         raise ValueError(f"All tensors must have same dtype, got A:{A.dtype}, B:{B.dtype}, C:{C.dtype}")
-    require_gpu_tensors(shmem, A=A, B=B, C=C)
-
     workspace = matmul_reduce_scatter_preamble(shmem, C, A, B, config, workspace)
     if stage is not None:
         stage(workspace)
@@ -139,6 +137,7 @@ def matmul_reduce_scatter(
     elif scale_a is not None or scale_b is not None:
         raise ValueError("scale_a / scale_b only apply to float8 inputs")
 
+    require_gpu_tensors(shmem, A=A, B=B, C=C)
     iris_launch(
         "iris_hip_matmul_reduce_scatter",
         grid,

@@ -1,0 +1,166 @@
+"""The five BASELINE configurations at full size on the GPU, against the CPU oracle.
+
+Inputs are drawn on the CPU from torch.Generator().manual_seed(seed) as the configurations state.
+Full-size comparisons use the oracle directly where it finishes in seconds; the largest case (fp8,
+16384 x 8192) is checked on row blocks plus size-independent properties (flags all raised, aux equal
+to the own product, untouched slots untouched).
+"""
+
+import pytest
+import torch
+
+import iris_amd as iris
+from iris_amd import _lib, ops
+from helpers import assert_bits_equal, heap_tensor, oracle, randn_cpu, slot_copies, stage_peers
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_plumbing_fp32_one_shot():
+    """fp32 256^3, uniform[-1,1] seed 0, one synthetic peer N(0,1) seed 1, W = 2, one-shot."""
+    g = torch.Generator().manual_seed(0)
+    A = torch.rand((256, 256), generator=g) * 2 - 1
+    B = torch.rand((256, 256), generator=g) * 2 - 1
+    peer = randn_cpu((256, 256), 1, torch.float32)
+    ctx = iris.iris(1 << 26, num_ranks=2, rank=0)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((256, 256), dtype=torch.float32)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="one_shot")
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    stage_peers(ctx, ws, [None, peer])
+    ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws)
+    exp = oracle.matmul_all_reduce(A, B, [None, peer], 0, 2, 64, 64, "one_shot")
+    assert oracle.rel_frobenius(dC.cpu(), exp["C"][0]) <= 1e-5
+    assert torch.allclose(dC.cpu(), A @ B + peer, atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+def test_config2_matmul_all_reduce_bf16(variant):
+    M, N, K, W = 4096, 4096, 1376, 8
+    g = torch.Generator().manual_seed(0)
+    A = (torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16)
+    B = (torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16)
+    peers = [None] + [randn_cpu((M, N), r, torch.bfloat16) for r in range(1, W)]
+    ctx = iris.iris(1 << 28, num_ranks=W, rank=0)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=torch.bfloat16)
+    cfg = iris.FusedConfig(all_reduce_variant=variant)  # 256 x 64 flag tiles: 1024 flags
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    assert ws.locks.numel() == 1024
+    stage_peers(ctx, ws, peers)
+    ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws)
+    kernel = _lib.last_kernel()
+    assert kernel.startswith("mfma_bf16_256x256"), kernel
+    exp = oracle.matmul_all_reduce(A, B, peers, 0, W, 256, 64, variant)
+    assert torch.all(ws.locks.cpu() == 1)
+    assert oracle.rel_frobenius(ws.aux_buffer.cpu(), exp["aux"]) <= 1e-2
+    got = slot_copies(ctx, dC)
+    for r in range(W):
+        assert oracle.rel_frobenius(got[r], exp["C"][r]) <= 1e-2, f"slot {r}"
+    # The slot sum itself must be exact given the aux the kernel produced.
+    again = oracle.slot_sum(ws.aux_buffer.cpu(), peers[1:])
+    if variant == "one_shot":
+        assert_bits_equal(got[0], again, "slot sum from the kernel's own aux")
+        for r in range(1, W):
+            assert torch.all(got[r] == 0)
+    else:
+        mine = torch.from_numpy(oracle.owner_map(M, N, 256, 64, W, "two_shot") == 0)
+        for r in range(W):
+            assert_bits_equal(got[r], torch.where(mine, again, torch.zeros_like(again)), f"slot {r}")
+
+
+def test_config3_all_gather_matmul_bf16_rows():
+    W, M_local, K, N = 8, 1024, 4096, 1792
+    shards = [(randn_cpu((M_local, K), r, torch.float32) / K ** 0.5).to(torch.bfloat16) for r in range(W)]
+    B = (randn_cpu((K, N), 8, torch.float32) / K ** 0.5).to(torch.bfloat16)
+    ctx = iris.iris(1 << 27, num_ranks=W, rank=0)
+    dA = ctx.zeros((M_local, K), dtype=torch.bfloat16)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    out = ctx.zeros((W * M_local, N), dtype=torch.bfloat16)
+    ops.all_gather_matmul(ctx, out, dA, dB, gather_dim=0)
+    assert _lib.last_kernel().startswith("mfma_bf16"), _lib.last_kernel()
+    ref = oracle.all_gather_matmul(shards, B, gather_dim=0)
+    assert oracle.rel_frobenius(out.cpu(), ref) <= 1e-2
+
+
+def test_config3_shape_in_reference_layout_columns():
+    """The same GEMM shape in the reference's layout: A sharded along K (K_local = 512)."""
+    W, M, K_local, N = 8, 8192, 512, 1792
+    K = W * K_local
+    shards = [(randn_cpu((M, K_local), r, torch.float32) / K ** 0.5).to(torch.bfloat16) for r in range(W)]
+    B = (randn_cpu((K, N), 8, torch.float32) / K ** 0.5).to(torch.bfloat16)
+    ctx = iris.iris(1 << 27, num_ranks=W, rank=2)
+    dA = ctx.zeros((M, K_local), dtype=torch.bfloat16)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    out = ctx.zeros((M, N), dtype=torch.bfloat16)
+    ops.all_gather_matmul(ctx, out, dA, dB)
+    assert oracle.rel_frobenius(out.cpu(), oracle.all_gather_matmul(shards, B)) <= 1e-2
+
+
+def test_config4_matmul_reduce_scatter_bf16():
+    M, N, K, W = 8192, 4096, 1376, 8
+    g = torch.Generator().manual_seed(0)
+    A = (torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16)
+    B = (torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16)
+    ctx = iris.iris(1 << 28, num_ranks=W, rank=0)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=torch.bfloat16)
+    for r in range(W):
+        ctx.peer_view(dC, r).zero_()
+    ws = ops.matmul_reduce_scatter(ctx, dC, dA, dB, all_owners=True, sum_peers=False)
+    assert ws.locks.numel() == 2048 and torch.all(ws.locks.cpu() == 1)
+    ref = oracle.gemm(A, B)
+    aux = ws.aux_buffer.cpu()
+    assert oracle.rel_frobenius(aux, ref) <= 1e-2
+    got = slot_copies(ctx, dC)
+    for r in range(W):
+        rows = slice(1024 * r, 1024 * (r + 1))
+        assert_bits_equal(got[r][rows], aux[rows], f"row block {r} in slot {r}")
+        other = torch.ones(M, dtype=torch.bool)
+        other[rows] = False
+        assert torch.all(got[r][other] == 0), f"slot {r} holds rows it does not own"
+
+
+def _fp8_case(M, N, K, W, block_m):
+    a, b = randn_cpu((M, K), 0, torch.float32), randn_cpu((K, N), 1, torch.float32)
+    Aq, sa = oracle.quantize_e4m3(a)
+    Bq, sb = oracle.quantize_e4m3(b)
+    ctx = iris.iris(1 << 30, num_ranks=W, rank=0)
+    dA, dB = heap_tensor(ctx, Aq), heap_tensor(ctx, Bq)
+    dC = ctx.zeros((M, N), dtype=torch.bfloat16)
+    cfg = iris.FusedConfig(block_size_m=block_m, block_size_n=64, block_size_k=64, all_reduce_variant="one_shot")
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for r in range(1, W):
+        ctx.peer_view(ws.aux_buffer, r).copy_(torch.randn((M, N), generator=gen, device="cuda").to(torch.bfloat16))
+        ctx.peer_view(ws.locks, r).fill_(1)
+    ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, scale_a=sa, scale_b=sb)
+    return ctx, ws, dC, Aq, Bq, sa * sb, _lib.last_kernel()
+
+
+def test_config5a_fp8_matmul_all_reduce():
+    M, N, K, W = 16384, 8192, 1024, 8
+    ctx, ws, dC, Aq, Bq, scale, kernel = _fp8_case(M, N, K, W, 256)
+    assert kernel.startswith("mfma_fp8_256x256"), kernel
+    assert torch.all(ws.locks.cpu() == 1)
+    for r0 in (0, 5120, M - 256):
+        rows = slice(r0, r0 + 256)
+        own = oracle.gemm(Aq[rows], Bq, torch.bfloat16, scale)
+        aux = ws.aux_buffer[rows].cpu()
+        assert oracle.rel_frobenius(aux, own) <= 3e-2
+        peers = [ctx.peer_view(ws.aux_buffer, r)[rows].cpu() for r in range(1, W)]
+        assert_bits_equal(dC[rows].cpu(), oracle.slot_sum(aux, peers), f"rows {r0}")
+
+
+def test_config5b_fp8_skinny():
+    M, N, K, W = 32, 8192, 1024, 8
+    ctx, ws, dC, Aq, Bq, scale, kernel = _fp8_case(M, N, K, W, 32)
+    own = oracle.gemm(Aq, Bq, torch.bfloat16, scale)
+    aux = ws.aux_buffer.cpu()
+    assert oracle.rel_frobenius(aux, own) <= 3e-2, kernel
+    peers = [ctx.peer_view(ws.aux_buffer, r).cpu() for r in range(1, W)]
+    assert_bits_equal(dC.cpu(), oracle.slot_sum(aux, peers), kernel)

@@ -1,0 +1,345 @@
+"""GPU parity tests: the HIP path, called through the package and the C ABI, against the CPU oracle.
+
+Tolerances (relative Frobenius error): 1e-2 for bfloat16/float16/float32, 3e-2 for float8 inputs.
+Flags, owners, destinations and - for integer-valued inputs, where the fp32 product is exact -
+every output bit must match.
+"""
+
+import pytest
+import torch
+
+import iris_amd as iris
+from iris_amd import _lib
+from iris_amd import ops
+from helpers import (assert_bits_equal, heap_tensor, oracle, randint_cpu, randn_cpu, slot_copies, stage_peers)
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 1e-2, torch.float16: 1e-2, torch.float32: 1e-2}
+HEAP = 1 << 28
+
+
+def _ctx(world, rank=0, heap=HEAP):
+    return iris.iris(heap, num_ranks=world, rank=rank)
+
+
+def _run_all_reduce(ctx, A, B, peers, cfg, mode="fp32", path="auto", out_dtype=None, **kw):
+    out_dtype = out_dtype or A.dtype
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((A.shape[0], B.shape[1]), dtype=out_dtype)
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    if peers is not None:
+        stage_peers(ctx, ws, peers)
+    ws = ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, slot_sum=mode, kernel_path=path, **kw)
+    return dC, ws, _lib.last_kernel()
+
+
+# ------------------------------------------------------------------------------------------------
+# W = 1: every operator is a plain GEMM (the reference's own single-rank test configuration)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(128, 64, 32), (1024, 256, 512), (256, 256, 64), (512, 384, 1376)])
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+def test_single_rank_is_gemm(dtype, M, N, K, variant):
+    ctx = _ctx(1)
+    A, B = randn_cpu((M, K), 0, dtype), randn_cpu((K, N), 1, dtype)
+    small = M <= 128 or K <= 64 or N <= 128 or dtype == torch.float32
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant=variant) if small \
+        else iris.FusedConfig(all_reduce_variant=variant)
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, None, cfg)
+    ref = oracle.gemm(A, B)
+    err = oracle.rel_frobenius(dC.cpu(), ref)
+    assert err <= TOL[dtype], f"{kernel}: rel Frobenius {err}"
+    # the reference's own acceptance test (tests/ops/test_matmul_all_reduce.py:18-25,89)
+    atol, rtol = {torch.float16: (0.2, 0.01), torch.float32: (0.3, 0.01), torch.bfloat16: (2.5, 0.02)}[dtype]
+    assert torch.allclose(dC.cpu().float(), ref.float(), atol=atol, rtol=rtol)
+    assert torch.all(ws.locks.cpu() == 1)
+    assert_bits_equal(ws.aux_buffer.cpu(), dC.cpu(), "aux vs C at W=1")
+    if dtype != torch.float32:
+        assert kernel.startswith("mfma"), kernel
+
+
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_exact_inputs_bit_exact(path, dtype):
+    """Integer-valued inputs make the fp32 product exact, so the whole output must match bit for bit."""
+    ctx = _ctx(1)
+    M, N, K = 384, 320, 160
+    A, B = randint_cpu((M, K), 3, dtype), randint_cpu((K, N), 4, dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="one_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, None, cfg, path=path)
+    assert kernel.startswith(path)
+    assert_bits_equal(dC.cpu(), oracle.gemm(A, B), f"{kernel} exact GEMM")
+
+
+# ------------------------------------------------------------------------------------------------
+# W = 8 all-reduce: slot sums, flags, owners, destinations
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+@pytest.mark.parametrize("mode", ["fp32", "reference"])
+@pytest.mark.parametrize("rank", [0, 5])
+def test_all_reduce_bit_exact(path, variant, mode, rank):
+    W, dtype = 8, torch.bfloat16
+    M, N, K = 512, 384, 96
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 10, dtype), randint_cpu((K, N), 11, dtype)
+    peers = [randn_cpu((M, N), 100 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=128, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg, mode=mode, path=path)
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, 128, 64, variant, mode)
+    assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], "aux")
+    assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+    got = slot_copies(ctx, dC)
+    for r in range(W):
+        assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
+
+
+def test_all_reduce_closed_form():
+    """Rank r contributes r + 1 everywhere: every element sums to W(W+1)/2
+    (the reference's tile-collective check, tests/context/test_all_reduce.py:245-246,352-356)."""
+    W, dtype = 8, torch.bfloat16
+    M, N, K = 256, 256, 64
+    for rank in (0, 3):
+        ctx = _ctx(W, rank)
+        A = torch.zeros(M, K, dtype=dtype)
+        A[:, 0] = rank + 1
+        B = torch.zeros(K, N, dtype=dtype)
+        B[0, :] = 1
+        peers = [torch.full((M, N), float(r + 1), dtype=dtype) for r in range(W)]
+        cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="one_shot")
+        dC, ws, _ = _run_all_reduce(ctx, A, B, peers, cfg)
+        assert torch.all(dC.cpu().float() == W * (W + 1) / 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_all_reduce_random(dtype):
+    W, rank = 4, 1
+    M, N, K = 1024, 256, 512
+    ctx = _ctx(W, rank)
+    A, B = randn_cpu((M, K), 0, dtype, K ** -0.5), randn_cpu((K, N), 1, dtype)
+    peers = [randn_cpu((M, N), 7 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="two_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg)
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, 64, 64, "two_shot")
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert oracle.rel_frobenius(got, exp["C"][r]) <= TOL[dtype], f"{kernel} slot {r}"
+    mine = torch.from_numpy(oracle.owner_map(M, N, 64, 64, W, "two_shot") == rank)
+    assert torch.all(dC.cpu()[~mine] == 0), "tiles of other owners must stay untouched"
+
+
+def test_flag_tiles_larger_than_kernel_tiles():
+    """Flag tiles that span several kernel tiles are raised exactly once, by the last arrival."""
+    W, rank, dtype = 2, 0, torch.bfloat16
+    M, N, K = 1024, 1024, 64
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 1, dtype), randint_cpu((K, N), 2, dtype)
+    peers = [randn_cpu((M, N), 50 + r, dtype) for r in range(W)]
+    for bm, bn in [(512, 512), (384, 200), (1024, 1024)]:
+        cfg = iris.FusedConfig(block_size_m=bm, block_size_n=bn, block_size_k=32, all_reduce_variant="one_shot")
+        dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg)
+        exp = oracle.matmul_all_reduce(A, B, peers, rank, W, bm, bn, "one_shot")
+        assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), f"{kernel} flags {bm}x{bn}"
+        assert_bits_equal(dC.cpu(), exp["C"][rank], f"{kernel} {bm}x{bn}")
+
+
+@pytest.mark.parametrize("M,N,K", [(100, 72, 50), (130, 66, 33), (257, 129, 70)])
+def test_ragged_shapes_generic(M, N, K):
+    W, rank, dtype = 3, 2, torch.float16
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 5, dtype), randint_cpu((K, N), 6, dtype)
+    peers = [randn_cpu((M, N), 20 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=32, block_size_n=24, block_size_k=16, all_reduce_variant="two_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg)
+    assert kernel.startswith("generic")
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, 32, 24, "two_shot")
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert_bits_equal(got, exp["C"][r], f"slot {r}")
+    assert torch.all(ws.locks.cpu() == 1)
+
+
+def test_transposed_b_and_strided_views():
+    """B handed over as the transpose of an (N, K) tensor (K-contiguous) takes the MFMA path too."""
+    ctx = _ctx(1)
+    dtype = torch.bfloat16
+    M, N, K = 256, 384, 128
+    A, Bt = randint_cpu((M, K), 8, dtype), randint_cpu((N, K), 9, dtype)
+    dA, dBt = heap_tensor(ctx, A), heap_tensor(ctx, Bt)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="one_shot")
+    ops.matmul_all_reduce(ctx, dC, dA, dBt.t(), config=cfg)
+    assert _lib.last_kernel().endswith("_nt"), _lib.last_kernel()
+    assert_bits_equal(dC.cpu(), oracle.gemm(A, Bt.t()), "NT GEMM")
+
+
+# ------------------------------------------------------------------------------------------------
+# reduce-scatter
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("rank", [0, 7])
+def test_reduce_scatter_bit_exact(path, rank):
+    W, dtype = 8, torch.bfloat16
+    M, N, K = 640, 256, 64   # 10 x 4 tiles of 64x64 = 40 tiles: 5 per rank
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 12, dtype), randint_cpu((K, N), 13, dtype)
+    peers = [randn_cpu((M, N), 200 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    ws = ops.matmul_reduce_scatter(ctx, dC, dA, dB, config=cfg, kernel_path=path,
+                                   stage=lambda w: stage_peers(ctx, w, peers))
+    exp = oracle.matmul_reduce_scatter(A, B, peers, rank, W, 64, 64)
+    assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], "aux")
+    assert torch.all(ws.locks.cpu() == 1)
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert_bits_equal(got, exp["C"][r], f"C in slot {r}")
+
+
+def test_reduce_scatter_reference_acceptance():
+    """The reference's own check (tests/ops/test_matmul_reduce_scatter.py:24-89) at W = 1."""
+    for dtype, atol, rtol in [(torch.float16, 2e-1, 1e-2), (torch.float32, 1e-1, 1e-2)]:
+        ctx = _ctx(1)
+        M, N, K = 128, 128, 32
+        A, B = randn_cpu((M, K), 0, dtype), randn_cpu((K, N), 1, dtype)
+        dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+        dC = ctx.zeros((M, N), dtype=dtype)
+        cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32)
+        ops.matmul_reduce_scatter(ctx, dC, dA, dB, config=cfg)
+        assert torch.allclose(dC.cpu().float(), (A.float() @ B.float()), atol=atol, rtol=rtol)
+
+
+def test_reduce_scatter_all_owners_row_blocks():
+    """One launch standing in for all ranks: row block r lands in slot r at its global coordinates."""
+    W, rank, dtype = 8, 0, torch.bfloat16
+    M, N, K = 2048, 512, 64   # 256x64 tiles: 8 x 8 = 64 tiles, 8 per rank = one tile row = 256 rows
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 14, dtype), randint_cpu((K, N), 15, dtype)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dC, r).zero_()
+    ops.matmul_reduce_scatter(ctx, dC, dA, dB, all_owners=True, sum_peers=False)
+    exp = oracle.matmul_reduce_scatter(A, B, None, rank, W, 256, 64, all_owners=True, sum_peers=False)
+    full = oracle.gemm(A, B)
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert_bits_equal(got, exp["C"][r], f"slot {r}")
+        assert_bits_equal(got[256 * r:256 * (r + 1)], full[256 * r:256 * (r + 1)], f"row block {r}")
+
+
+# ------------------------------------------------------------------------------------------------
+# all-gather + matmul
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("M,K_local,N", [(128, 32, 64), (256, 64, 128), (512, 96, 256)])
+@pytest.mark.parametrize("W", [1, 2, 8])
+def test_all_gather_matmul_columns(path, M, K_local, N, W):
+    dtype, rank = torch.float16, W - 1
+    ctx = _ctx(W, rank)
+    shards = [randint_cpu((M, K_local), 42 + r, dtype) for r in range(W)]
+    B = randint_cpu((W * K_local, N), 123, dtype)
+    dA = ctx.zeros((M, K_local), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    out = ctx.zeros((M, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32)
+    ops.all_gather_matmul(ctx, out, dA, dB, config=cfg, kernel_path=path)
+    assert _lib.last_kernel().startswith(path)
+    assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B), _lib.last_kernel())
+
+
+def test_all_gather_matmul_rows_and_bias():
+    W, rank, dtype = 8, 3, torch.bfloat16
+    M_local, K, N = 128, 256, 192
+    ctx = _ctx(W, rank)
+    shards = [randint_cpu((M_local, K), 60 + r, dtype) for r in range(W)]
+    B = randint_cpu((K, N), 70, dtype)
+    bias = randint_cpu((W * M_local,), 71, dtype, -8, 9)
+    dA = ctx.zeros((M_local, K), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB, dbias = heap_tensor(ctx, B), heap_tensor(ctx, bias)
+    out = ctx.zeros((W * M_local, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32)
+    for path in ("mfma", "generic"):
+        out.zero_()
+        ops.all_gather_matmul(ctx, out, dA, dB, bias=dbias, config=cfg, gather_dim=0, kernel_path=path)
+        assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B, bias=bias, gather_dim=0), path)
+
+
+def test_all_gather_matmul_random_via_namespace():
+    W, rank, dtype = 4, 0, torch.float16
+    M, K_local, N = 256, 64, 128
+    ctx = _ctx(W, rank)
+    shards = [randn_cpu((M, K_local), 42 + r, dtype) for r in range(W)]
+    B = randn_cpu((W * K_local, N), 123, dtype)
+    dA = ctx.zeros((M, K_local), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    out = ctx.zeros((M, N), dtype=dtype)
+    ctx.ops.all_gather_matmul(out, dA, dB, config=iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32))
+    ref = torch.cat(shards, dim=1).float() @ B.float()
+    # tests/ops/test_all_gather_matmul.py:97-101: atol = rtol = 1e-2 for fp16 ... on fp16-rounded reference
+    assert torch.allclose(out.cpu().float(), ref.half().float(), atol=5e-2, rtol=1e-2)
+    assert oracle.rel_frobenius(out.cpu(), ref) <= 1e-2
+
+
+# ------------------------------------------------------------------------------------------------
+# float8 inputs
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (32, 512, 256), (512, 384, 192)])
+def test_fp8_all_reduce(path, M, N, K):
+    W, rank = 8, 0
+    ctx = _ctx(W, rank)
+    a, b = randn_cpu((M, K), 0, torch.float32), randn_cpu((K, N), 1, torch.float32)
+    Aq, sa = oracle.quantize_e4m3(a)
+    Bq, sb = oracle.quantize_e4m3(b)
+    peers = [randn_cpu((M, N), 30 + r, torch.bfloat16) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=32, block_size_n=64, block_size_k=64, all_reduce_variant="one_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, Aq, Bq, peers, cfg, path=path, out_dtype=torch.bfloat16, scale_a=sa, scale_b=sb)
+    assert kernel.startswith(path), kernel
+    exp = oracle.matmul_all_reduce(Aq, Bq, peers, rank, W, 32, 64, "one_shot", out_dtype=torch.bfloat16, scale=sa * sb)
+    assert oracle.rel_frobenius(ws.aux_buffer.cpu(), exp["aux"]) <= 3e-2
+    assert oracle.rel_frobenius(dC.cpu(), exp["C"][rank]) <= 3e-2
+    # against the unquantised product the error is the quantisation error, still within the bound
+    assert oracle.rel_frobenius(ws.aux_buffer.cpu(), a @ b) <= 6e-2
+
+
+# ------------------------------------------------------------------------------------------------
+# protocol and error behaviour
+# ------------------------------------------------------------------------------------------------
+def test_unstaged_peer_flags_time_out():
+    """A peer that never raises its flags: the kernel gives up after spin_limit polls and the next
+    barrier reports it (the reference would spin forever, iris/mem/triton/context.py:758)."""
+    W, rank, dtype = 2, 0, torch.bfloat16
+    ctx = _ctx(W, rank)
+    ctx.spin_limit = 64
+    M, N, K = 256, 256, 64
+    dA, dB = heap_tensor(ctx, randint_cpu((M, K), 1, dtype)), heap_tensor(ctx, randint_cpu((K, N), 2, dtype))
+    dC = ctx.zeros((M, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="one_shot")
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    ctx.peer_view(ws.locks, 1).zero_()
+    with pytest.raises(RuntimeError, match="peer flag"):
+        ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws)
+    assert torch.all(ws.locks.cpu() == 1), "own flags are raised before waiting"
+
+
+def test_c_abi_rejects_bad_arguments():
+    lib = _lib.library()
+    import ctypes
+    ctx = _ctx(1)
+    t = ctx.zeros((64, 64), dtype=torch.bfloat16)
+    null = ctypes.c_void_p(0)
+    p = ctypes.c_void_p(t.data_ptr())
+    rc = lib.iris_hip_matmul_all_reduce(p, p, p, null, null, 64, 64, 64, 64, 1, 64, 1, 64, 1, null, 0, 1, 64, 64, 32,
+                                        _lib.VARIANT_ONE_SHOT, _lib.BF16, _lib.BF16, 1.0, 0, 0, null, 0, null)
+    assert rc == 1 and "aux_buffer" in _lib.last_error()
+    rc = lib.iris_hip_matmul_all_reduce(p, p, p, p, p, 64, 64, 64, 64, 1, 64, 1, 64, 1, null, 0, 1, 64, 64, 32,
+                                        7, _lib.BF16, _lib.BF16, 1.0, 0, 0, null, 0, null)
+    assert rc == 1 and "variant" in _lib.last_error()
+    cu, xcc, lds = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int32()
+    assert lib.iris_hip_query(0, ctypes.byref(cu), ctypes.byref(xcc), ctypes.byref(lds)) == 0
+    assert cu.value == torch.cuda.get_device_properties(0).multi_processor_count and xcc.value >= 1
