@@ -1,0 +1,322 @@
+#!/usr/bin/env python3
+"""Benchmark of the rank-local fused GEMM+collective path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Prints ONE JSON line.  A step is one launch of the fused operator on synthetic inputs that already
+sit in HBM (peers' partial results and flags staged before the timed region).  `value` is the
+whole-job throughput of the K timed steps in TFLOP/s (2*M*N*K flop per step); `roofline` prices the
+same launches, timed one by one with GPU events on the launch stream, against the roof that bounds
+the fused kernel (HBM for the slot-sum workloads, MFMA for the others); `gemm_phase` repeats the
+measurement with the peers switched off (W = 1), which isolates the MFMA phase; `cpu_baseline` times
+torch's CPU matmul plus the slot reduction on a bounded sample of the same workload.
+
+Default workload: BASELINE configuration 2, matmul_all_reduce bf16 M=N=4096, K=1376, W=8.
+"""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s")}
+
+
+def _randn(shape, seed, dtype, scale=1.0, device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * scale).to(dtype)
+
+
+class Workload:
+    """One configuration: builds the heap tensors, launches a step, knows its flop and byte counts."""
+
+    name = ""
+    dtype = "bf16"
+    bound = "hbm"
+
+    def setup(self, iris, world):
+        raise NotImplementedError
+
+    def step(self):
+        raise NotImplementedError
+
+
+class MatmulAllReduce(Workload):
+    def __init__(self, name, M, N, K, fp8=False, block_m=256, variant="one_shot"):
+        self.name, self.M, self.N, self.K, self.fp8 = name, M, N, K, fp8
+        self.block_m, self.variant = block_m, variant
+        self.dtype = "fp8" if fp8 else "bf16"
+        self.flops = 2 * M * N * K
+
+    def algorithmic_bytes(self, world):
+        es = 1 if self.fp8 else 2
+        return self.M * self.K * es + self.K * self.N * es + (world - 1) * self.M * self.N * 2 + self.M * self.N * 2
+
+    def describe(self, world):
+        return {"workload": self.name, "op": "matmul_all_reduce", "variant": self.variant, "M": self.M, "N": self.N,
+                "K": self.K, "W": world, "flag_tile": [self.block_m, 64]}
+
+    def setup(self, iris, world):
+        from iris_amd import ops
+        M, N, K = self.M, self.N, self.K
+        heap = 4 * M * N + 2 * (M * K + K * N) + (64 << 20)
+        self.ctx = ctx = iris.iris(heap, num_ranks=world, rank=0)
+        self.scale = {}
+        if self.fp8:
+            a, b = _randn((M, K), 0, torch.float32), _randn((K, N), 1, torch.float32)
+            sa, sb = float(a.abs().max()) / 448.0, float(b.abs().max()) / 448.0
+            A, B = (a / sa).to(torch.float8_e4m3fn), (b / sb).to(torch.float8_e4m3fn)
+            self.scale = dict(scale_a=sa, scale_b=sb)
+        else:
+            g = torch.Generator().manual_seed(0)
+            A = (torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16)
+            B = (torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16)
+        self.A_cpu, self.B_cpu = A, B
+        self.A = ctx.zeros((M, K), dtype=A.dtype)
+        self.A.copy_(A)
+        self.B = ctx.zeros((K, N), dtype=B.dtype)
+        self.B.copy_(B)
+        self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
+        self.cfg = iris.FusedConfig(block_size_m=self.block_m, block_size_n=64, block_size_k=64,
+                                    all_reduce_variant=self.variant)
+        self.ws = ops.matmul_all_reduce_preamble(ctx, self.C, self.A, self.B, config=self.cfg)
+        gen = torch.Generator(device="cuda").manual_seed(1)
+        for r in range(1, world):  # synthetic peer partials, N(0,1) in bf16, flags raised
+            ctx.peer_view(self.ws.aux_buffer, r).copy_(
+                torch.randn((M, N), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16))
+            ctx.peer_view(self.ws.locks, r).fill_(1)
+        self._op = ops.matmul_all_reduce
+        torch.cuda.synchronize()
+
+    def step(self):
+        # The flags and aux written by the previous step are simply overwritten: no reset is needed.
+        self.ws.prepared = True
+        self._op(self.ctx, self.C, self.A, self.B, async_op=True, config=self.cfg, workspace=self.ws, **self.scale)
+
+    def cpu_baseline(self, world, budget_s=20.0):
+        """torch CPU matmul (bf16 in, as the GPU path; fp8 dequantised to fp32) + slot reduction, on
+        the first rows of the workload."""
+        rows = min(self.M, 1024)
+        A = self.A_cpu[:rows]
+        A = A.float() if self.fp8 else A
+        B = self.B_cpu.float() if self.fp8 else self.B_cpu
+        peers = [_randn((rows, self.N), 100 + r, torch.bfloat16) for r in range(1, world)]
+
+        def once():
+            C = torch.matmul(A, B).to(torch.bfloat16)
+            acc = C.float()
+            for p in peers:
+                acc += p.float()
+            return acc.to(torch.bfloat16)
+
+        once()
+        times, t_end = [], time.perf_counter() + budget_s
+        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+            t0 = time.perf_counter()
+            once()
+            times.append(time.perf_counter() - t0)
+        t = statistics.median(times)
+        return {"value": 2 * rows * self.N * self.K / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                "kind": "port", "sample": f"first {rows} of {self.M} rows, {len(times)} reps, median; "
+                                          f"torch.matmul + fp32 sum of {world} slots; os.cpu_count={os.cpu_count()}"}
+
+
+class AllGatherMatmul(Workload):
+    bound = "bf16"
+
+    def __init__(self, name, M, N, K):
+        self.name, self.M, self.N, self.K = name, M, N, K
+        self.flops = 2 * M * N * K
+
+    def algorithmic_bytes(self, world):
+        return 2 * (self.M * self.K + self.K * self.N + self.M * self.N)
+
+    def describe(self, world):
+        return {"workload": self.name, "op": "all_gather_matmul", "gather": "rows", "M": self.M, "N": self.N,
+                "K": self.K, "W": world}
+
+    def setup(self, iris, world):
+        from iris_amd import ops
+        M, N, K = self.M, self.N, self.K
+        self.ctx = ctx = iris.iris(2 * (M // world * K + K * N + M * N) + (64 << 20), num_ranks=world, rank=0)
+        self.A = ctx.zeros((M // world, K), dtype=torch.bfloat16)
+        for r in range(world):
+            ctx.peer_view(self.A, r).copy_(_randn((M // world, K), r, torch.bfloat16, K ** -0.5))
+        self.B = ctx.zeros((K, N), dtype=torch.bfloat16)
+        self.B.copy_(_randn((K, N), 8, torch.bfloat16, K ** -0.5))
+        self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
+        self._op = ops.all_gather_matmul
+        torch.cuda.synchronize()
+
+    def step(self):
+        self._op(self.ctx, self.C, self.A, self.B, async_op=True, gather_dim=0)
+
+    def cpu_baseline(self, world, budget_s=20.0):
+        return None
+
+
+class MatmulReduceScatter(Workload):
+    bound = "bf16"
+
+    def __init__(self, name, M, N, K):
+        self.name, self.M, self.N, self.K = name, M, N, K
+        self.flops = 2 * M * N * K
+
+    def algorithmic_bytes(self, world):
+        return 2 * (self.M * self.K + self.K * self.N + self.M * self.N)
+
+    def describe(self, world):
+        return {"workload": self.name, "op": "matmul_reduce_scatter", "M": self.M, "N": self.N, "K": self.K,
+                "W": world, "all_owners": True, "sum_peers": False}
+
+    def setup(self, iris, world):
+        from iris_amd import _lib
+        from iris_amd.ops import FusedConfig, matmul_reduce_scatter_preamble
+        from iris_amd.ops._common import current_stream, iris_launch, ptr
+        M, N, K = self.M, self.N, self.K
+        self.ctx = ctx = iris.iris(2 * (M * K + K * N + 2 * M * N) + (64 << 20), num_ranks=world, rank=0)
+        g = torch.Generator().manual_seed(0)
+        self.A = ctx.zeros((M, K), dtype=torch.bfloat16)
+        self.A.copy_((torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16))
+        self.B = ctx.zeros((K, N), dtype=torch.bfloat16)
+        self.B.copy_((torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16))
+        self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
+        cfg = FusedConfig()
+        ws = matmul_reduce_scatter_preamble(ctx, self.C, self.A, self.B, cfg)
+        A, B, C = self.A, self.B, self.C
+        # The operator wrapper re-runs its preamble (two barriers, three memsets) on every call, as
+        # the reference does; the step times the launch alone, through the same C entry point.
+        self._launch = lambda: iris_launch(
+            "iris_hip_matmul_reduce_scatter", (ws.locks.numel(),),
+            ptr(A), ptr(B), ptr(C), ptr(ws.aux_buffer), ptr(ws.locks), M, N, K,
+            A.stride(0), A.stride(1), B.stride(0), B.stride(1), C.stride(0), C.stride(1),
+            ptr(ctx.get_device_context()), 0, world, cfg.block_size_m, cfg.block_size_n, cfg.block_size_k,
+            1, 0, _lib.BF16, _lib.BF16, 1.0, _lib.ACC_FP32, ctx.spin_limit, ptr(ctx._status), _lib.PATH_AUTO,
+            current_stream(ctx), algorithm="matmul_reduce_scatter", rank=0)
+        torch.cuda.synchronize()
+
+    def step(self):
+        self._launch()
+
+    def cpu_baseline(self, world, budget_s=20.0):
+        return None
+
+
+WORKLOADS = {
+    "matmul_all_reduce_bf16_4096x4096x1376": lambda: MatmulAllReduce("matmul_all_reduce_bf16_4096x4096x1376", 4096, 4096, 1376),
+    "matmul_all_reduce_two_shot_bf16_4096x4096x1376": lambda: MatmulAllReduce(
+        "matmul_all_reduce_two_shot_bf16_4096x4096x1376", 4096, 4096, 1376, variant="two_shot"),
+    "all_gather_matmul_bf16_8192x1792x4096": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096", 8192, 1792, 4096),
+    "matmul_reduce_scatter_bf16_8192x4096x1376": lambda: MatmulReduceScatter("matmul_reduce_scatter_bf16_8192x4096x1376", 8192, 4096, 1376),
+    "matmul_all_reduce_fp8_16384x8192x1024": lambda: MatmulAllReduce("matmul_all_reduce_fp8_16384x8192x1024", 16384, 8192, 1024, fp8=True),
+    "matmul_all_reduce_fp8_skinny_32x8192x1024": lambda: MatmulAllReduce(
+        "matmul_all_reduce_fp8_skinny_32x8192x1024", 32, 8192, 1024, fp8=True, block_m=32),
+}
+DEFAULT = "matmul_all_reduce_bf16_4096x4096x1376"
+
+
+def timed_steps(wl, steps, warmup):
+    """W untimed steps, then K timed ones between device synchronisations; every timed launch is also
+    bracketed by GPU events on the launch stream."""
+    for _ in range(warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        wl.step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    wl.ctx.check_status()
+    per_launch_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    return wall, per_launch_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--world", type=int, default=8, help="number of heap slots W")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-gemm-phase", action="store_true", help="skip the W=1 measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build runs the rank-local path of one MI355X "
+                 "(the W ranks are heap slots in its HBM); --gpus must be 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+
+    import iris_amd as iris
+    from iris_amd import _lib
+
+    wl = WORKLOADS[args.workload]()
+    wl.setup(iris, args.world)
+    wall, per_launch_ms = timed_steps(wl, args.steps, args.warmup)
+    kernel = _lib.last_kernel()
+    ms_per_step = wall * 1e3 / args.steps
+    launch_ms = statistics.mean(per_launch_ms)
+    tflops = wl.flops * args.steps / wall / 1e12
+
+    bytes_alg = wl.algorithmic_bytes(args.world)
+    if wl.bound == "hbm":
+        peak, unit = PEAK["hbm"]
+        achieved = bytes_alg / (launch_ms * 1e-3) / 1e9
+    else:
+        peak, unit = PEAK[wl.dtype]
+        achieved = wl.flops / (launch_ms * 1e-3) / 1e12
+    roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "achieved": round(achieved, 2), "peak": peak,
+                "unit": unit, "frac": round(achieved / peak, 4), "traffic": None, "kernel": kernel,
+                "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(per_launch_ms), 5),
+                "algorithmic_bytes": bytes_alg, "algorithmic_flops": wl.flops}
+
+    out = {
+        "metric": "TFLOP/s and % of MI355X MFMA peak, rank-local fused GEMM+epilogue, 1 GPU",
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl.dtype,
+        "data": "synthetic",
+        "config": wl.describe(args.world),
+        "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2),
+        "roofline": roofline,
+    }
+
+    if isinstance(wl, MatmulAllReduce) and not args.no_gemm_phase:
+        del wl.ctx, wl
+        torch.cuda.empty_cache()
+        solo = WORKLOADS[args.workload]()
+        solo.setup(iris, 1)  # W = 1: same kernel and shape, no peers to sum
+        wall1, per1 = timed_steps(solo, args.steps, args.warmup)
+        t1 = solo.flops * args.steps / wall1 / 1e12
+        out["gemm_phase"] = {"world": 1, "tflops": round(t1, 3), "ms_per_step": round(wall1 * 1e3 / args.steps, 5),
+                             "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4), "kernel": _lib.last_kernel()}
+        wl = solo
+
+    if not args.no_cpu:
+        base = wl.cpu_baseline(args.world)
+        if base is not None:
+            base["value"] = round(base["value"], 4)
+            out["cpu_baseline"] = base
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
