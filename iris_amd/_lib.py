@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIBRARY_PATH = os.path.join(_HERE, "lib", "libiris_hip.so")
+# IRIS_HIP_LIBRARY names another build of the same library (e.g. one compiled with other tile shapes).
+LIBRARY_PATH = os.environ.get("IRIS_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libiris_hip.so")
 
 ABI_VERSION = 1
 

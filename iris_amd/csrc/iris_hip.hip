@@ -200,10 +200,13 @@ struct MfmaCfg {
   static constexpr int LA = A_BYTES / kDmaBytes / NW;  // direct-to-LDS loads per thread per K step
   static constexpr int LB = B_BYTES / kDmaBytes / NW;
   static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
-  // Epilogue staging: one 32-row slab of the wave's block, 16-bit elements, padded rows.
-  static constexpr int SROW = TN * 2 + 16;
-  static constexpr int STG_BYTES = 32 * SROW;
-  static constexpr int SMEM_BYTES = RING_BYTES > NW * STG_BYTES ? RING_BYTES : NW * STG_BYTES;
+  // Epilogue staging: the whole output tile in 16-bit elements, rows padded by 16 bytes so that
+  // the accumulator-layout writes (one row per lane) spread over the LDS banks.
+  static constexpr int TROW = BN * 2 + 16;
+  static constexpr int TILE_BYTES = BM * TROW;
+  static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES;
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+  static_assert(NT % (BN / 8) == 0 && BM % (NT / (BN / 8)) == 0, "epilogue pass shape");
   static_assert(A_BYTES % (kDmaBytes * NW) == 0 && B_BYTES % (kDmaBytes * NW) == 0, "tile/loader mismatch");
   static_assert(BK % KM == 0 && TM % 32 == 0 && TN % 32 == 0, "tile/MFMA mismatch");
   static_assert(STAGES >= 3, "the ring needs at least three slots");
@@ -434,7 +437,6 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
   const int klocal = (p.gather == GATHER_K) ? p.K_local : p.K;
   const int nkb = cdiv(klocal, BK);
   const int nsteps = nsrc * nkb;
-  char* const stg = smem + wave * CFG::STG_BYTES;
   const unsigned smem_base = __builtin_amdgcn_readfirstlane(lds_address(smem));
   const unsigned long long a_own = (unsigned long long)p.A;
 
@@ -564,55 +566,63 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     __syncthreads();
 
     // ---- epilogue -------------------------------------------------------------------------------
-    const int wrow0 = m0 + wm * TM;  // first row / column of this wave's block
-    const int wcol0 = n0 + wn * TN;
-    constexpr int CPR = TN / 8;      // 16-byte chunks per staged row
-    constexpr int RPI = 64 / CPR;    // staged rows covered by one wave-wide access
-    constexpr int ITERS = 32 / RPI;
-    const int rd_row = lane / CPR, rd_chunk = lane % CPR;
-    const int ftn = cdiv(p.N, p.flag_bn);
-    const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
-
-    // Write slab mb (32 rows of the wave's block) to the wave's staging area as 16-bit elements.
-    auto stage_slab = [&](int mb, const f32x16_t (&blk)[NB]) {
-      float badd = 0.f;
-      if (p.bias) {
-        const int gm = wrow0 + mb * 32 + acc_col(lane);
-        if (gm < p.M) badd = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
+    // The whole output tile is first written to LDS in the output type (the operand ring is dead
+    // by now), which frees the accumulators; both phases then stream rows of the tile, 16 bytes per
+    // lane and BN*2 contiguous bytes per row, with many loads in flight per thread.
+    {
+      float badd[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        badd[mb] = 0.f;
+        if (p.bias) {
+          const int gm = m0 + wm * TM + mb * 32 + acc_col(lane);
+          if (gm < p.M) badd[mb] = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
+        }
       }
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          unsigned short h[4];
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = Out::from_float(acc_read(blk[nb][4 * q + e]) * p.scale + badd);
-          u32x2_t w;
-          w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
-          w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
-          const int ncol = nb * 32 + acc_row(lane, 4 * q);
-          *(LDS_AS u32x2_t*)(LDS_AS char*)(stg + acc_col(lane) * CFG::SROW + ncol * 2) = w;
-        }
-      __builtin_amdgcn_wave_barrier();
-    };
+          for (int q = 0; q < 4; ++q) {
+            unsigned short h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              h[e] = Out::from_float(acc_read(acc.v[mb][nb][4 * q + e]) * p.scale + badd[mb]);
+            u32x2_t w;
+            w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
+            w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+            const int trow = wm * TM + mb * 32 + acc_col(lane);
+            const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
+            *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
+          }
+    }
+    __syncthreads();
+
+    constexpr int CPR = BN / 8;            // 16-byte chunks per tile row
+    constexpr int RPP = NT / CPR;          // tile rows covered by one pass of the workgroup
+    constexpr int PASSES = BM / RPP;
+    const int t_row = tid / CPR, t_chunk = tid % CPR;
+    const int gn = n0 + t_chunk * 8;
+    const bool col_ok = gn < p.N;
+    const char* const t_lds = smem + t_row * CFG::TROW + t_chunk * 16;
 
     // Phase 1: C (plain store) or aux (own slot).
-    char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      stage_slab(mb, acc.v[mb]);
-#pragma unroll
-      for (int i = 0; i < ITERS; ++i) {
-        const int r = i * RPI + rd_row;
-        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(stg + r * CFG::SROW + rd_chunk * 16);
-        const int gm = wrow0 + mb * 32 + r, gn = wcol0 + rd_chunk * 8;
-        if (gm < p.M && gn < p.N) *(u32x4_t*)(out1 + ((long long)gm * p.s_cm + gn) * 2) = v;
+    {
+      char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+#pragma unroll 4
+      for (int ps = 0; ps < PASSES; ++ps) {
+        const int gm = m0 + ps * RPP + t_row;
+        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + ps * RPP * CFG::TROW);
+        if (gm < p.M && col_ok) *(u32x4_t*)(out1 + ((long long)gm * p.s_cm + gn) * 2) = v;
       }
-      __builtin_amdgcn_wave_barrier();
     }
 
     if (p.epi != EPI_STORE) {
-      __atomic_thread_fence(__ATOMIC_RELEASE);  // system scope: the aux stores precede the flags
+      // Publish: every wave waits until its aux stores have reached L2, the workgroup meets, and
+      // the threads that raise flags do so with system-scope release (one L2 write-back per
+      // workgroup instead of one per wave).
+      wait_vmcnt<0>();
       __syncthreads();
       raise_flags<BM, BN, NT>(p, m0, n0, tid);
       if (p.sum_peers && p.world > 1) {
@@ -623,67 +633,74 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       // Phase 2: reduce the flag tiles this rank is responsible for.
       const bool ref_chain = (p.acc_mode == IRIS_HIP_ACC_REFERENCE) && !Out::kFp32SumInReference;
       const unsigned long long aux_own = (unsigned long long)p.aux, c_own = (unsigned long long)p.C;
+      const int ftn = cdiv(p.N, p.flag_bn);
+      const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+      const int fcol = gn / p.flag_bn;
+      const bool peers_cached = p.sum_peers && p.world <= kMaxCachedSlots;
+      constexpr int G = 2;  // passes whose peer loads are issued together
+      static_assert(PASSES % G == 0, "pass grouping");
+
+      for (int pg = 0; pg < PASSES; pg += G) {
+        bool active[G];
+        long long eoff[G];
+        int owner[G];
+        u32x4_t pv[G][kMaxCachedSlots];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        stage_slab(mb, acc.v[mb]);
-#pragma unroll 2
-        for (int i = 0; i < ITERS; ++i) {
-          const int r = i * RPI + rd_row;
-          const u32x4_t own = *(const LDS_AS u32x4_t*)(LDS_AS char*)(stg + r * CFG::SROW + rd_chunk * 16);
-          const int gm = wrow0 + mb * 32 + r, gn = wcol0 + rd_chunk * 8;
-          if (!(gm < p.M && gn < p.N)) continue;
-          const int t = (gm / p.flag_bm) * ftn + gn / p.flag_bn;
-          const int owner = owner_of(p.epi, t, ftotal, p.world, p.rank);
-          if (!p.all_owners && owner != p.rank) continue;
-          const long long eoff = ((long long)gm * p.s_cm + gn) * 2;
+        for (int g = 0; g < G; ++g) {
+          const int gm = m0 + (pg + g) * RPP + t_row;
+          active[g] = gm < p.M && col_ok;
+          const int t = (gm / p.flag_bm) * ftn + fcol;
+          owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+          if (!p.all_owners && owner[g] != p.rank) active[g] = false;
+          eoff[g] = ((long long)gm * p.s_cm + gn) * 2;
+          if (active[g] && peers_cached) {
+#pragma unroll
+            for (int j = 0; j < kMaxCachedSlots; ++j)
+              if (j < p.world && j != p.rank) pv[g][j] = *(const u32x4_t*)(hb[j] + (aux_own - hb_own) + eoff[g]);
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if (!active[g]) continue;
+          const u32x4_t own = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
           float sum[8];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             sum[2 * e] = Out::to_float((unsigned short)(own[e] & 0xFFFF));
             sum[2 * e + 1] = Out::to_float((unsigned short)(own[e] >> 16));
           }
-          if (p.sum_peers) {
-            for (int rb0 = 0; rb0 < p.world; rb0 += kMaxCachedSlots) {
-              u32x4_t pv[kMaxCachedSlots];
+          auto add_peer = [&](const u32x4_t& v) {
 #pragma unroll
-              for (int j = 0; j < kMaxCachedSlots; ++j) {
-                const int pr = rb0 + j;
-                if (pr < p.world && pr != p.rank) {
-                  const unsigned long long base = (rb0 == 0 ? hb[j] : (unsigned long long)p.heap_bases[pr]) + (aux_own - hb_own);
-                  pv[j] = *(const u32x4_t*)(base + eoff);
-                }
-              }
-#pragma unroll
-              for (int j = 0; j < kMaxCachedSlots; ++j) {
-                const int pr = rb0 + j;
-                if (pr < p.world && pr != p.rank) {
-#pragma unroll
-                  for (int e = 0; e < 4; ++e) {
-                    sum[2 * e] += Out::to_float((unsigned short)(pv[j][e] & 0xFFFF));
-                    sum[2 * e + 1] += Out::to_float((unsigned short)(pv[j][e] >> 16));
-                  }
-                  if (ref_chain) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
-                  }
-                }
-              }
+            for (int e = 0; e < 4; ++e) {
+              sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
+              sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
             }
+            if (ref_chain) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
+            }
+          };
+          if (peers_cached) {
+#pragma unroll
+            for (int j = 0; j < kMaxCachedSlots; ++j)
+              if (j < p.world && j != p.rank) add_peer(pv[g][j]);
+          } else if (p.sum_peers) {
+            for (int pr = 0; pr < p.world; ++pr)
+              if (pr != p.rank) add_peer(*(const u32x4_t*)(in_slot(aux_own, pr) + eoff[g]));
           }
           u32x4_t res;
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
           if (p.epi == EPI_TWO_SHOT) {
-            *(u32x4_t*)(c_own + eoff) = res;
+            *(u32x4_t*)(c_own + eoff[g]) = res;
             for (int pr = 0; pr < p.world; ++pr)
-              if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff) = res;
+              if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
           } else {
-            const int dst = p.all_owners ? owner : p.rank;
-            *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff) = res;
+            const int dst = p.all_owners ? owner[g] : p.rank;
+            *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]) = res;
           }
         }
-        __builtin_amdgcn_wave_barrier();
       }
     }
     // Staging shares LDS with the operand ring of the next tile.
