@@ -26,6 +26,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "iris_hip.h"
 #include "layout.h"
 
@@ -630,77 +632,94 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
         __syncthreads();
       }
 
-      // Phase 2: reduce the flag tiles this rank is responsible for.
+      // Phase 2: reduce the flag tiles this rank is responsible for.  The peer loads are issued
+      // unconditionally (rows this thread does not reduce read the tile origin instead) and for a
+      // compile-time number of peers, so that all loads of a group of passes are in flight
+      // together; only the stores are predicated.
       const bool ref_chain = (p.acc_mode == IRIS_HIP_ACC_REFERENCE) && !Out::kFp32SumInReference;
       const unsigned long long aux_own = (unsigned long long)p.aux, c_own = (unsigned long long)p.C;
       const int ftn = cdiv(p.N, p.flag_bn);
       const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
       const int fcol = gn / p.flag_bn;
-      const bool peers_cached = p.sum_peers && p.world <= kMaxCachedSlots;
-      constexpr int G = 2;  // passes whose peer loads are issued together
-      static_assert(PASSES % G == 0, "pass grouping");
+      const int npeers = p.sum_peers ? p.world - 1 : 0;
+      // Peer aux bases in ascending rank order, own rank skipped.
+      unsigned long long pb[kMaxCachedSlots - 1];
+#pragma unroll
+      for (int i = 0; i < kMaxCachedSlots - 1; ++i) pb[i] = (i < p.rank ? hb[i] : hb[i + 1]) + (aux_own - hb_own);
+      const long long safe_off = ((long long)m0 * p.s_cm + n0) * 2;  // first element of the tile
 
-      for (int pg = 0; pg < PASSES; pg += G) {
-        bool active[G];
-        long long eoff[G];
-        int owner[G];
-        u32x4_t pv[G][kMaxCachedSlots];
+      auto reduce_tile = [&](auto np_tag) {
+        constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
+        constexpr int NPV = NP > 0 ? NP : 1;
+        constexpr int G = NP >= 4 ? 2 : 4;           // passes whose loads are issued together
+        static_assert(PASSES % G == 0, "pass grouping");
+        for (int pg = 0; pg < PASSES; pg += G) {
+          bool active[G];
+          long long eoff[G];
+          int owner[G];
+          u32x4_t own[G], pv[G][NPV];
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const int gm = m0 + (pg + g) * RPP + t_row;
-          active[g] = gm < p.M && col_ok;
-          const int t = (gm / p.flag_bm) * ftn + fcol;
-          owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
-          if (!p.all_owners && owner[g] != p.rank) active[g] = false;
-          eoff[g] = ((long long)gm * p.s_cm + gn) * 2;
-          if (active[g] && peers_cached) {
+          for (int g = 0; g < G; ++g) {
+            const int gm = m0 + (pg + g) * RPP + t_row;
+            const int t = (gm / p.flag_bm) * ftn + fcol;
+            owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+            active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
+            eoff[g] = active[g] ? ((long long)gm * p.s_cm + gn) * 2 : safe_off;
+            if constexpr (NP > 0) {
 #pragma unroll
-            for (int j = 0; j < kMaxCachedSlots; ++j)
-              if (j < p.world && j != p.rank) pv[g][j] = *(const u32x4_t*)(hb[j] + (aux_own - hb_own) + eoff[g]);
+              for (int i = 0; i < NP; ++i) pv[g][i] = *(const u32x4_t*)(pb[i] + eoff[g]);
+            }
+            own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
           }
-        }
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-          if (!active[g]) continue;
-          const u32x4_t own = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
-          float sum[8];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sum[2 * e] = Out::to_float((unsigned short)(own[e] & 0xFFFF));
-            sum[2 * e + 1] = Out::to_float((unsigned short)(own[e] >> 16));
-          }
-          auto add_peer = [&](const u32x4_t& v) {
+          for (int g = 0; g < G; ++g) {
+            float sum[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
-              sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
+              sum[2 * e] = Out::to_float((unsigned short)(own[g][e] & 0xFFFF));
+              sum[2 * e + 1] = Out::to_float((unsigned short)(own[g][e] >> 16));
             }
-            if (ref_chain) {
+            auto add_peer = [&](const u32x4_t& v) {
 #pragma unroll
-              for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
+              for (int e = 0; e < 4; ++e) {
+                sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
+                sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
+              }
+              if (ref_chain) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
+              }
+            };
+            if constexpr (NP > 0) {
+#pragma unroll
+              for (int i = 0; i < NP; ++i) add_peer(pv[g][i]);
+            } else if constexpr (NP < 0) {
+              for (int pr = 0; pr < p.world; ++pr)
+                if (pr != p.rank) add_peer(*(const u32x4_t*)(in_slot(aux_own, pr) + eoff[g]));
             }
-          };
-          if (peers_cached) {
+            u32x4_t res;
 #pragma unroll
-            for (int j = 0; j < kMaxCachedSlots; ++j)
-              if (j < p.world && j != p.rank) add_peer(pv[g][j]);
-          } else if (p.sum_peers) {
-            for (int pr = 0; pr < p.world; ++pr)
-              if (pr != p.rank) add_peer(*(const u32x4_t*)(in_slot(aux_own, pr) + eoff[g]));
-          }
-          u32x4_t res;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
-          if (p.epi == EPI_TWO_SHOT) {
-            *(u32x4_t*)(c_own + eoff[g]) = res;
-            for (int pr = 0; pr < p.world; ++pr)
-              if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
-          } else {
-            const int dst = p.all_owners ? owner[g] : p.rank;
-            *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]) = res;
+            for (int e = 0; e < 4; ++e)
+              res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
+            if (active[g]) {
+              if (p.epi == EPI_TWO_SHOT) {
+                *(u32x4_t*)(c_own + eoff[g]) = res;
+                for (int pr = 0; pr < p.world; ++pr)
+                  if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
+              } else {
+                const int dst = p.all_owners ? owner[g] : p.rank;
+                *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]) = res;
+              }
+            }
           }
         }
+      };
+      switch (p.world <= kMaxCachedSlots ? npeers : -1) {
+        case 0: reduce_tile(std::integral_constant<int, 0>{}); break;
+        case 1: reduce_tile(std::integral_constant<int, 1>{}); break;
+        case 3: reduce_tile(std::integral_constant<int, 3>{}); break;
+        case 7: reduce_tile(std::integral_constant<int, 7>{}); break;
+        default: reduce_tile(std::integral_constant<int, -1>{}); break;
       }
     }
     // Staging shares LDS with the operand ring of the next tile.
