@@ -109,7 +109,6 @@ def all_gather_matmul(
         raise ValueError(
             f"All tensors must have same dtype, got A:{A_sharded.dtype}, B:{B.dtype}, C:{output_tensor.dtype}"
         )
-    require_gpu_tensors(shmem, A_sharded=A_sharded, B=B, output_tensor=output_tensor, bias=bias)
     if not shmem.is_symmetric(A_sharded):
         raise RuntimeError("A_sharded must be allocated on the symmetric heap (the peers' shards are read by offset)")
 
@@ -133,6 +132,8 @@ def all_gather_matmul(
     elif scale_a is not None or scale_b is not None:
         raise ValueError("scale_a / scale_b only apply to float8 inputs")
 
+    path = path_code(kernel_path)
+    require_gpu_tensors(shmem, A_sharded=A_sharded, B=B, output_tensor=output_tensor, bias=bias)
     num_sms = config.num_sms if config.num_sms is not None else shmem.get_cu_count()
     iris_launch(
         "iris_hip_all_gather_matmul",
@@ -144,7 +145,7 @@ def all_gather_matmul(
         config.block_size_m, config.block_size_n, config.block_size_k,
         _lib.GATHER_K if gather_dim == 1 else _lib.GATHER_M,
         dtype_code(A_sharded.dtype), dtype_code(output_tensor.dtype), bias_code, scale,
-        path_code(kernel_path), current_stream(shmem),
+        path, current_stream(shmem),
         algorithm="all_gather_matmul",
         rank=rank,
         dtype=A_sharded.dtype,

@@ -165,6 +165,7 @@ def matmul_all_reduce(
     elif scale_a is not None or scale_b is not None:
         raise ValueError("scale_a / scale_b only apply to float8 inputs")
 
+    acc, path = acc_code(slot_sum), path_code(kernel_path)
     require_gpu_tensors(shmem, A=A, B=B, C=C)
     iris_launch(
         "iris_hip_matmul_all_reduce",
@@ -175,8 +176,8 @@ def matmul_all_reduce(
         ptr(device_context), rank, world_size,
         config.block_size_m, config.block_size_n, config.block_size_k,
         _VARIANT_CODES[config.all_reduce_variant],
-        dtype_code(A.dtype), dtype_code(C.dtype), scale, acc_code(slot_sum),
-        shmem.spin_limit, ptr(shmem._status), path_code(kernel_path), current_stream(shmem),
+        dtype_code(A.dtype), dtype_code(C.dtype), scale, acc,
+        shmem.spin_limit, ptr(shmem._status), path, current_stream(shmem),
         algorithm="matmul_all_reduce",
         rank=rank,
         dtype=A.dtype,

@@ -137,6 +137,7 @@ def matmul_reduce_scatter(
     elif scale_a is not None or scale_b is not None:
         raise ValueError("scale_a / scale_b only apply to float8 inputs")
 
+    acc, path = acc_code(slot_sum), path_code(kernel_path)
     require_gpu_tensors(shmem, A=A, B=B, C=C)
     iris_launch(
         "iris_hip_matmul_reduce_scatter",
@@ -147,8 +148,8 @@ def matmul_reduce_scatter(
         ptr(shmem.get_device_context()), rank, world_size,
         config.block_size_m, config.block_size_n, config.block_size_k,
         int(bool(all_owners)), int(bool(sum_peers)),
-        dtype_code(A.dtype), dtype_code(C.dtype), scale, acc_code(slot_sum),
-        shmem.spin_limit, ptr(shmem._status), path_code(kernel_path), current_stream(shmem),
+        dtype_code(A.dtype), dtype_code(C.dtype), scale, acc,
+        shmem.spin_limit, ptr(shmem._status), path, current_stream(shmem),
         algorithm="matmul_reduce_scatter",
         rank=rank,
         dtype=A.dtype,

@@ -1,0 +1,252 @@
+// Host-side check of iris_amd/csrc/layout.h: replays, on the CPU, what the gfx950 kernels do with the
+// index functions - direct-to-LDS deposits, 16-byte fragment reads, LDS transpose reads - and checks
+// that every MFMA operand slot receives the element the kernel assumes, that the LDS swizzles are
+// bijections without bank conflicts inside a 16-lane group, and that the tile orders and flag-tile
+// counts are exact.  The transpose-read semantics used here (within each 16-lane group, output lane i
+// element e comes from input lane 4e + i/4, element i%4 for 16-bit data; input lane 2e + i/8, byte
+// i%8 for 8-bit data) were measured on an MI355X.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <set>
+#include <vector>
+
+#include "layout.h"
+
+using namespace iris_layout;
+
+static int failures = 0;
+#define CHECK(cond, ...)                         \
+  do {                                           \
+    if (!(cond)) {                               \
+      if (failures < 20) { printf("FAIL %s:%d: ", __FILE__, __LINE__); printf(__VA_ARGS__); printf("\n"); } \
+      ++failures;                                \
+    }                                            \
+  } while (0)
+
+// ---- swizzle bijection + bank spread -------------------------------------------------------------
+template <int RB>
+void check_row_tile(int rows) {
+  using T = RowTile<RB>;
+  std::set<int> seen;
+  for (int r = 0; r < rows; ++r)
+    for (int c = 0; c < T::kChunksPerRow; ++c) {
+      int off = T::lds_offset(r, c);
+      CHECK(off >= 0 && off < rows * RB && off % 16 == 0, "row tile offset out of range");
+      CHECK(seen.insert(off).second, "row tile offset reused");
+      int r2, c2;
+      T::from_lds(off, r2, c2);
+      CHECK(r2 == r && c2 == c, "row tile inverse mismatch RB=%d r=%d c=%d", RB, r, c);
+    }
+  // 16 lanes reading the same logical chunk of 16 consecutive rows: 16 distinct 16-byte bank groups
+  for (int r0 = 0; r0 + 16 <= rows; r0 += 16)
+    for (int c = 0; c < T::kChunksPerRow; ++c) {
+      std::set<int> banks;
+      for (int i = 0; i < 16; ++i) banks.insert((T::lds_offset(r0 + i, c) % 256) / 16);
+      CHECK(banks.size() == 16, "row tile RB=%d bank conflict at rows %d.., chunk %d (%zu groups)", RB, r0, c, banks.size());
+    }
+}
+
+template <int RB, int ES>
+void check_col_tile(int krows) {
+  using T = ColTile<RB, ES>;
+  std::set<int> seen;
+  for (int k = 0; k < krows; ++k)
+    for (int c = 0; c < T::kChunksPerRow; ++c) {
+      int off = T::lds_offset(k, c);
+      CHECK(off >= 0 && off < krows * RB, "col tile offset out of range");
+      CHECK(seen.insert(off).second, "col tile offset reused");
+      int k2, c2;
+      T::from_lds(off, k2, c2);
+      CHECK(k2 == k && c2 == c, "col tile inverse mismatch");
+    }
+}
+
+// ---- simulate loader + fragment reads for one operand tile -----------------------------------------
+// Element identity: (row-or-k, col) packed in an int; the simulated LDS stores one id per element.
+struct Lds {
+  std::vector<int> id;  // per byte/ES element slot
+  int es;
+  Lds(int bytes, int es_) : id(bytes / es_, -1), es(es_) {}
+  int& at(int byte_off) { return id[byte_off / es]; }
+};
+
+// K-contiguous operand (A, or B^T): tile [rows][BK], fragment lanes per frag16_*/frag8_*.
+template <int RB, int ES>
+void sim_row_operand(int rows, int nwaves) {
+  using T = RowTile<RB>;
+  const int CE = 16 / ES, BK = RB / ES;
+  Lds lds(rows * RB, ES);
+  // loader: wave w, instruction i deposits 1 KiB at (w + i*nwaves)*1024; lane l its 16 bytes
+  const int ninstr = rows * RB / kDmaBytes;
+  for (int q = 0; q < ninstr; ++q)
+    for (int lane = 0; lane < 64; ++lane) {
+      int off = q * kDmaBytes + lane * 16, row, c;
+      T::from_lds(off, row, c);
+      for (int e = 0; e < CE; ++e) lds.at(off + e * ES) = row * 4096 + (c * CE + e);  // global (row, k)
+    }
+  for (int x : lds.id) CHECK(x >= 0, "row operand: LDS element never written");
+  // fragment reads: block of 32 rows starting at r0, every k-slice
+  const int KM = ES == 2 ? 16 : 64;
+  for (int r0 = 0; r0 + 32 <= rows; r0 += 32)
+    for (int kk = 0; kk < BK / KM; ++kk)
+      for (int lane = 0; lane < 64; ++lane) {
+        const int nfrag = ES == 2 ? 1 : 2;
+        for (int h = 0; h < nfrag; ++h) {
+          int c = ES == 2 ? frag16_chunk(lane, kk) : frag8_chunk(lane, kk, h);
+          int off = T::lds_offset(r0 + frag16_row(lane), c);
+          for (int e = 0; e < CE; ++e) {
+            int got = lds.at(off + e * ES);
+            // MFMA slot: row lane%32, k = kk*KM + (KM/2)*(lane/32) + h*CE + e
+            int want = (r0 + lane % 32) * 4096 + kk * KM + (KM / 2) * (lane / 32) + h * CE + e;
+            CHECK(got == want, "row operand ES=%d lane %d kk %d: got (%d,%d) want (%d,%d)", ES, lane, kk, got / 4096, got % 4096, want / 4096, want % 4096);
+          }
+        }
+      }
+}
+
+// N-contiguous operand (row-major B): tile [BK][BN], transpose reads.
+template <int RB, int ES>
+void sim_col_operand(int BK) {
+  using T = ColTile<RB, ES>;
+  const int CE = 16 / ES, BN = RB / ES;
+  Lds lds(BK * RB, ES);
+  const int ninstr = BK * RB / kDmaBytes;
+  for (int q = 0; q < ninstr; ++q)
+    for (int lane = 0; lane < 64; ++lane) {
+      int off = q * kDmaBytes + lane * 16, k, c;
+      T::from_lds(off, k, c);
+      for (int e = 0; e < CE; ++e) lds.at(off + e * ES) = k * 4096 + (c * CE + e);  // global (k, n)
+    }
+  for (int x : lds.id) CHECK(x >= 0, "col operand: LDS element never written");
+  const int KM = ES == 2 ? 16 : 64;
+  const int per_read = ES == 2 ? 4 : 8;     // elements a lane contributes / receives per transpose read
+  const int nreads = ES == 2 ? 2 : 4;
+  for (int n0 = 0; n0 + 32 <= BN; n0 += 32)
+    for (int kk = 0; kk < BK / KM; ++kk)
+      for (int rd = 0; rd < nreads; ++rd) {
+        // every lane presents an address; the hardware redistributes within 16-lane groups
+        int addr[64];
+        std::set<int> banks_by_group[4];
+        for (int lane = 0; lane < 64; ++lane) {
+          int krow = ES == 2 ? tr16_krow(lane, kk, rd) : tr8_krow(lane, kk, rd);
+          int n = n0 + (ES == 2 ? tr16_ncol(lane) : tr8_ncol(lane));
+          addr[lane] = T::lds_offset(krow, n / CE) + (n % CE) * ES;
+          for (int b = 0; b < 8; b += 4) banks_by_group[lane / 16].insert(((addr[lane] + b) % 256) / 4);
+        }
+        for (int g = 0; g < 4; ++g)
+          CHECK(banks_by_group[g].size() == 32, "col operand ES=%d: bank conflict in lane group %d (%zu banks)", ES, g, banks_by_group[g].size());
+        for (int lane = 0; lane < 64; ++lane) {
+          int grp = lane / 16, i = lane % 16;
+          for (int e = 0; e < per_read; ++e) {
+            int src_lane = grp * 16 + (ES == 2 ? 4 * e + i / 4 : 2 * e + i / 8);
+            int src_elem = ES == 2 ? i % 4 : i % 8;
+            int got = lds.at(addr[src_lane] + src_elem * ES);
+            // MFMA slot of lane: n = lane%32, k = kk*KM + (KM/2)*(lane/32) + rd*per_read + e
+            int want = (kk * KM + (KM / 2) * (lane / 32) + rd * per_read + e) * 4096 + n0 + lane % 32;
+            CHECK(got == want, "col operand ES=%d lane %d kk %d read %d elem %d: got (k%d,n%d) want (k%d,n%d)", ES, lane, kk, rd, e,
+                  got / 4096, got % 4096, want / 4096, want % 4096);
+          }
+        }
+      }
+}
+
+// ---- accumulator layout: every (n, m) of a 32x32 block owned exactly once -----------------------------
+void check_acc_layout() {
+  std::set<int> seen;
+  for (int lane = 0; lane < 64; ++lane)
+    for (int i = 0; i < 16; ++i) {
+      int r = acc_row(lane, i), c = acc_col(lane);
+      CHECK(r >= 0 && r < 32 && c >= 0 && c < 32, "acc index range");
+      CHECK(seen.insert(r * 32 + c).second, "acc element owned twice");
+      if (i % 4) CHECK(acc_row(lane, i) == acc_row(lane, i - 1) + 1, "acc rows of a register quad must be consecutive");
+    }
+  CHECK(seen.size() == 1024, "acc layout must cover the block");
+}
+
+// ---- tile orders ---------------------------------------------------------------------------------------
+void check_tile_orders() {
+  for (int tm = 1; tm <= 40; tm += 3)
+    for (int tn = 1; tn <= 40; tn += 5)
+      for (int g : {1, 2, 4, 8, 16}) {
+        std::set<int> seen;
+        for (int idx = 0; idx < tm * tn; ++idx) {
+          int a, b;
+          grouped_tile(idx, tm, tn, g, a, b);
+          CHECK(a >= 0 && a < tm && b >= 0 && b < tn, "grouped_tile out of range tm=%d tn=%d g=%d idx=%d -> (%d,%d)", tm, tn, g, idx, a, b);
+          seen.insert(a * tn + b);
+        }
+        CHECK((int)seen.size() == tm * tn, "grouped_tile is not a bijection tm=%d tn=%d g=%d", tm, tn, g);
+      }
+  for (int total : {1, 7, 8, 10, 224, 255, 256, 257, 1000, 2048})
+    for (int nwg : {1, 5, 8, 16, 224, 256})
+      for (int xcd : {1, 8}) {
+        std::map<int, int> count;
+        for (int wg = 0; wg < nwg; ++wg) {
+          bool ended = false;
+          for (int it = 0; it < total + 2; ++it) {
+            int idx = xcd_tile_index(wg, nwg, it, total, xcd);
+            if (idx < 0) { ended = true; continue; }
+            CHECK(!ended, "xcd_tile_index resumed after it ended (total=%d nwg=%d)", total, nwg);
+            CHECK(idx < total, "xcd_tile_index out of range");
+            count[idx]++;
+          }
+        }
+        CHECK((int)count.size() == total, "xcd_tile_index misses tiles: total=%d nwg=%d xcd=%d covered=%zu", total, nwg, xcd, count.size());
+        for (auto& kv : count) CHECK(kv.second == 1, "tile %d processed %d times", kv.first, kv.second);
+      }
+}
+
+// ---- flag tiles ----------------------------------------------------------------------------------------
+void check_flag_counts() {
+  struct Case { int M, N, FM, FN, KM, KN; };
+  for (Case c : {Case{4096, 4096, 256, 64, 256, 256}, Case{1024, 1024, 512, 512, 128, 128}, Case{1024, 1024, 384, 200, 128, 128},
+                 Case{100, 72, 32, 24, 64, 64}, Case{257, 129, 64, 64, 64, 64}, Case{1000, 600, 96, 96, 256, 256}}) {
+    int ftm = cdiv(c.M, c.FM), ftn = cdiv(c.N, c.FN);
+    for (int fm = 0; fm < ftm; ++fm)
+      for (int fn = 0; fn < ftn; ++fn) {
+        std::set<int> macro;
+        for (int m = fm * c.FM; m < (fm + 1) * c.FM && m < c.M; ++m)
+          for (int n = fn * c.FN; n < (fn + 1) * c.FN && n < c.N; n += 1) macro.insert((m / c.KM) * 100000 + n / c.KN);
+        int got = macro_tiles_over_flag_tile(fm, fn, c.FM, c.FN, c.KM, c.KN, c.M, c.N);
+        CHECK(got == (int)macro.size(), "macro_tiles_over_flag_tile(%d,%d) = %d, brute force %zu", fm, fn, got, macro.size());
+      }
+  }
+  for (int world : {1, 2, 3, 4, 8})
+    for (int total : {1, 4, 7, 40, 64, 2048}) {
+      int per = total / world;
+      for (int t = 0; t < total; ++t) {
+        int want = -1;
+        for (int r = 0; r < world; ++r) {
+          int s = r * per, e = (r == world - 1) ? total : s + per;
+          if (t >= s && t < e) want = r;
+        }
+        CHECK(owner_contiguous(t, total, world) == want, "owner_contiguous(%d,%d,%d)", t, total, world);
+        CHECK(owner_interleaved(t, world) == t % world, "owner_interleaved");
+      }
+    }
+}
+
+int main() {
+  check_row_tile<64>(256);
+  check_row_tile<128>(256);
+  check_row_tile<256>(64);
+  check_col_tile<512, 2>(32);
+  check_col_tile<256, 2>(32);
+  check_col_tile<256, 1>(64);
+  check_col_tile<128, 1>(64);
+  sim_row_operand<64, 2>(256, 8);   // bf16/fp16 A tile 256 x 32
+  sim_row_operand<64, 2>(128, 4);
+  sim_row_operand<64, 1>(256, 8);   // fp8 A tile 256 x 64
+  sim_col_operand<512, 2>(32);      // bf16 B tile 32 x 256
+  sim_col_operand<256, 2>(32);      // bf16 B tile 32 x 128
+  sim_col_operand<256, 1>(64);      // fp8 B tile 64 x 256
+  sim_col_operand<128, 1>(64);      // fp8 B tile 64 x 128
+  check_acc_layout();
+  check_tile_orders();
+  check_flag_counts();
+  if (failures) { printf("%d check(s) failed\n", failures); return 1; }
+  printf("layout_sim: all checks passed\n");
+  return 0;
+}

@@ -1,0 +1,215 @@
+"""The CPU oracle against everything that pins it without the GPU: the golden index-math vectors,
+closed forms from the reference's tests, brute force on tiny inputs, and torch library routines.
+A mistake in the oracle (a dropped term, a swapped index, a wrong rounding point) fails one of these.
+"""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import oracle, randint_cpu, randn_cpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "index_math.json")))
+
+
+# -- index math against the golden vectors ---------------------------------------------------------
+@pytest.mark.parametrize("case", GOLDEN["ownership_reduce_scatter"], ids=lambda c: f"{c['M']}x{c['N']}_W{c['world']}")
+def test_reduce_scatter_ownership_matches_reference_tests(case):
+    M, N, bm, bn, W = case["M"], case["N"], case["block_m"], case["block_n"], case["world"]
+    tiles_m, tiles_n = oracle.tile_grid(M, N, bm, bn)
+    total = tiles_m * tiles_n
+    assert total == case["total_tiles"]
+    owners = [oracle.owner_reduce_scatter(t, total, W) for t in range(total)]
+    omap = oracle.owner_map(M, N, bm, bn, W, "reduce_scatter")
+    for rank_s, tiles in case["owned"].items():
+        rank = int(rank_s)
+        mine = [t for t in range(total) if owners[t] == rank]
+        if isinstance(tiles, dict):
+            assert len(mine) == tiles["count"]
+            assert mine[0] == tiles["first"][0] and mine[-1] == tiles["last"][0]
+            rows = np.where((omap == rank).any(axis=1))[0]
+            assert [int(rows.min()), int(rows.max()) + 1] == tiles["rows"]
+            checks = [tiles["first"], tiles["last"]]
+        else:
+            assert mine == [t[0] for t in tiles]
+            checks = tiles
+        for tile_id, r0, r1, c0, c1 in checks:
+            assert oracle.tile_bounds(tile_id, M, N, bm, bn) == (r0, r1, c0, c1)
+            assert (omap[r0:r1, c0:c1] == rank).all()
+    assert sorted(set(owners)) == sorted({o for o in owners})  # every tile has exactly one owner
+
+
+def test_config4_row_blocks():
+    """8192 x 4096 with 256 x 64 tiles and W = 8: rank r owns exactly rows [1024 r, 1024 (r + 1))."""
+    omap = oracle.owner_map(8192, 4096, 256, 64, 8, "reduce_scatter")
+    for r in range(8):
+        assert (omap[1024 * r:1024 * (r + 1)] == r).all()
+
+
+@pytest.mark.parametrize("case", GOLDEN["ownership_two_shot"], ids=lambda c: f"{c['M']}x{c['N']}_W{c['world']}")
+def test_two_shot_ownership(case):
+    total, W = case["total_tiles"], case["world"]
+    assert oracle.tile_grid(case["M"], case["N"], case["block_m"], case["block_n"]) == (
+        oracle.cdiv(case["M"], case["block_m"]), oracle.cdiv(case["N"], case["block_n"]))
+    for rank_s, tiles in case["owned"].items():
+        mine = [t for t in range(total) if oracle.owner_two_shot(t, W) == int(rank_s)]
+        assert mine[:24] == tiles and len(mine) == case["owned_count"][rank_s]
+
+
+def test_tile_id_is_row_major():
+    assert oracle.tile_id(0, 0, 7) == 0 and oracle.tile_id(0, 6, 7) == 6 and oracle.tile_id(1, 0, 7) == 7
+    assert oracle.tile_id(3, 2, 64) == 194
+    assert oracle.tile_bounds(194, 4096, 4096, 256, 64) == (768, 1024, 128, 192)
+    assert oracle.tile_bounds(11, 100, 72, 32, 24) == (96, 100, 48, 72)  # ragged last row of tiles
+
+
+def test_bump_allocator_offsets():
+    g = GOLDEN["bump_allocator"]
+    offsets, end = oracle.bump_offsets([tuple(r) for r in g["requests"]], g["alignment"])
+    assert offsets == g["offsets"] and end == g["end"]
+
+
+def test_context_tensor_and_translate():
+    g = GOLDEN["context_tensor"]
+    assert oracle.context_tensor(g["rank"], g["world"], g["heap_bases"]).tolist() == g["expected"]
+    for t in GOLDEN["translate"]:
+        assert oracle.translate(t["ptr"], t["from"], t["to"], t["heap_bases"]) == t["expected"]
+    # translation is its own inverse and the identity within a rank
+    bases = [1 << 40, 3 << 40, 2 << 40]
+    p = (1 << 40) + 12345
+    assert oracle.translate(oracle.translate(p, 0, 2, bases), 2, 0, bases) == p
+    assert oracle.translate(p, 0, 0, bases) == p
+
+
+# -- arithmetic --------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_gemm_against_brute_force(dtype):
+    A, B = randint_cpu((9, 7), 1, dtype), randint_cpu((7, 5), 2, dtype)
+    assert torch.equal(oracle.gemm(A, B).double(), oracle.gemm_bruteforce(A, B))
+    # an asymmetric case catches a transposed operand: A (2x3) @ B (3x4)
+    A = torch.tensor([[1., 2., 3.], [4., 5., 6.]], dtype=dtype)
+    B = torch.tensor([[1., 0., 2., 1.], [0., 1., 1., 0.], [3., 0., 0., 1.]], dtype=dtype)
+    assert oracle.gemm(A, B).tolist() == [[10., 2., 4., 4.], [22., 5., 13., 10.]]
+
+
+def test_gemm_rounds_once_from_fp32():
+    """The product is accumulated in fp32 and cast once: summing 512 copies of 1 + 2^-7 gives 516,
+    while a bf16 accumulator gets stuck at 512."""
+    K = 512
+    A = torch.full((1, K), 1.0 + 2 ** -7, dtype=torch.bfloat16)
+    B = torch.full((K, 1), 1.0, dtype=torch.bfloat16)
+    assert float(oracle.gemm(A, B)) == float(torch.tensor(K * (1.0 + 2 ** -7)).to(torch.bfloat16))
+    acc = torch.zeros((), dtype=torch.bfloat16)
+    for _ in range(K):
+        acc = (acc + A[0, 0]).to(torch.bfloat16)
+    assert float(acc) != float(oracle.gemm(A, B))  # the wrong (bf16-accumulated) answer differs
+    A32, B32 = randn_cpu((33, 65), 5, torch.float32), randn_cpu((65, 17), 6, torch.float32)
+    assert torch.allclose(oracle.gemm(A32, B32), torch.matmul(A32, B32), rtol=1e-5, atol=1e-5)
+
+
+def test_gemm_bias_is_per_row_and_scale_applies_before_cast():
+    A, B = randint_cpu((4, 6), 3, torch.float32), randint_cpu((6, 3), 4, torch.float32)
+    bias = torch.tensor([10., 20., 30., 40.])
+    assert torch.equal(oracle.gemm(A, B, bias=bias), A @ B + bias[:, None])
+    assert torch.equal(oracle.gemm(A, B, scale=0.5), (A @ B) * 0.5)
+
+
+@pytest.mark.parametrize("W", [c["world"] for c in GOLDEN["closed_form_all_reduce"]])
+@pytest.mark.parametrize("mode", ["fp32", "reference"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_slot_sum_closed_form(W, mode, dtype):
+    expected = {c["world"]: c["value"] for c in GOLDEN["closed_form_all_reduce"]}[W]
+    for rank in range(W):
+        own = torch.full((8, 8), float(rank + 1), dtype=dtype)
+        peers = [torch.full((8, 8), float(r + 1), dtype=dtype) for r in range(W) if r != rank]
+        assert torch.all(oracle.slot_sum(own, peers, mode) == expected)
+
+
+def test_slot_sum_modes_differ_where_they_should():
+    """1 + 2^-8 + 2^-8: exact in fp32 (-> 1 + 2^-7 in bf16) but each bf16 add ties back to 1."""
+    own = torch.tensor([1.0], dtype=torch.bfloat16)
+    peers = [torch.tensor([2.0 ** -8], dtype=torch.bfloat16)] * 2
+    assert float(oracle.slot_sum(own, peers, "fp32")) == 1.0 + 2 ** -7
+    assert float(oracle.slot_sum(own, peers, "reference")) == 1.0
+    # fp16 data is summed in fp32 under both rules (acc_dtype = fp32 iff fp16)
+    own16 = torch.tensor([1.0], dtype=torch.float16)
+    peers16 = [torch.tensor([2.0 ** -12], dtype=torch.float16)] * 2
+    assert float(oracle.slot_sum(own16, peers16, "reference")) == float(oracle.slot_sum(own16, peers16, "fp32"))
+    # order: own first, then peers ascending (fp32 addition is not associative)
+    a, b, c = torch.tensor([1e8]), torch.tensor([-1e8]), torch.tensor([1.0])
+    assert float(oracle.slot_sum(a, [b, c])) == 1.0 and float(oracle.slot_sum(a, [c, b])) == 0.0
+
+
+def test_quantize_e4m3():
+    x = torch.tensor([448.0, -224.0, 1.0, 0.0, 0.4])
+    q, s = oracle.quantize_e4m3(x)
+    assert s == 1.0 and q.dtype == torch.float8_e4m3fn
+    assert q.float().tolist()[:4] == [448.0, -224.0, 1.0, 0.0]
+    assert abs(float(q[4].float()) - 0.4) <= 0.4 * 2 ** -4  # 3 mantissa bits
+    q2, s2 = oracle.quantize_e4m3(x * 3)
+    assert s2 == 3.0 and torch.equal(q2.float(), q.float())
+
+
+# -- operators ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+def test_all_reduce_world_of_one_is_gemm(variant):
+    A, B = randn_cpu((64, 32), 0, torch.float16), randn_cpu((32, 48), 1, torch.float16)
+    out = oracle.matmul_all_reduce(A, B, [None], 0, 1, 32, 16, variant)
+    assert torch.equal(out["C"][0], oracle.gemm(A, B)) and torch.equal(out["aux"], out["C"][0])
+    assert out["locks"].tolist() == [1] * 6
+
+
+def test_all_reduce_matches_torch_sum_over_ranks():
+    """The reference's acceptance check: torch.matmul + all_reduce(SUM) (tests/ops/test_matmul_all_reduce.py:57-62)."""
+    W, M, N, K = 4, 64, 48, 32
+    As = [randn_cpu((M, K), 10 + r, torch.float32) for r in range(W)]
+    B = randn_cpu((K, N), 99, torch.float32)
+    partials = [a @ B for a in As]
+    total = sum(partials)
+    for rank in range(W):
+        out = oracle.matmul_all_reduce(As[rank], B, partials, rank, W, 32, 16, "one_shot")
+        assert torch.allclose(out["C"][rank], total, rtol=1e-5, atol=1e-5)
+        two = oracle.matmul_all_reduce(As[rank], B, partials, rank, W, 32, 16, "two_shot")
+        mine = torch.from_numpy(oracle.owner_map(M, N, 32, 16, W, "two_shot") == rank)
+        for r in range(W):
+            assert torch.allclose(two["C"][r][mine], total[mine], rtol=1e-5, atol=1e-5)
+            assert torch.all(two["C"][r][~mine] == 0)
+    # the union over ranks of what two-shot writes covers C exactly once
+    cover = sum((torch.from_numpy(oracle.owner_map(M, N, 32, 16, W, "two_shot") == r)).int() for r in range(W))
+    assert torch.all(cover == 1)
+
+
+def test_reduce_scatter_matches_reference_acceptance():
+    """tests/ops/test_matmul_reduce_scatter.py:73-89: each owned tile equals the all-reduced product."""
+    W, M, N, K, bm, bn = 4, 128, 128, 32, 64, 64
+    A, B = randn_cpu((M, K), 0, torch.float32), randn_cpu((K, N), 1, torch.float32)
+    partial = A @ B
+    case = [c for c in GOLDEN["ownership_reduce_scatter"] if (c["M"], c["world"]) == (128, 4)][0]
+    for rank in range(W):
+        out = oracle.matmul_reduce_scatter(A, B, [partial] * W, rank, W, bm, bn)
+        for tile_id, r0, r1, c0, c1 in case["owned"][str(rank)]:
+            assert torch.allclose(out["C"][rank][r0:r1, c0:c1], W * partial[r0:r1, c0:c1], rtol=1e-5, atol=1e-5)
+        other = torch.from_numpy(oracle.owner_map(M, N, bm, bn, W, "reduce_scatter") != rank)
+        assert torch.all(out["C"][rank][other] == 0)
+        for r in range(W):
+            if r != rank:
+                assert torch.all(out["C"][r] == 0)
+    allo = oracle.matmul_reduce_scatter(A, B, None, 0, W, bm, bn, all_owners=True, sum_peers=False)
+    assert torch.equal(sum(allo["C"]), oracle.gemm(A, B))  # the slots partition the product
+
+
+def test_all_gather_matmul_both_layouts():
+    W = 4
+    shards = [randint_cpu((6, 5), 42 + r, torch.float16) for r in range(W)]
+    B = randint_cpu((20, 7), 123, torch.float16)
+    assert torch.equal(oracle.all_gather_matmul(shards, B), (torch.cat(shards, 1).float() @ B.float()).half())
+    # K order: shard r multiplies rows [5r, 5r+5) of B
+    manual = sum(shards[r].float() @ B[5 * r:5 * r + 5].float() for r in range(W)).half()
+    assert torch.equal(oracle.all_gather_matmul(shards, B), manual)
+    B2 = randint_cpu((5, 7), 124, torch.float16)
+    rows = oracle.all_gather_matmul(shards, B2, gather_dim=0)
+    for r in range(W):
+        assert torch.equal(rows[6 * r:6 * r + 6], (shards[r].float() @ B2.float()).half())
