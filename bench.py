@@ -209,7 +209,37 @@ class MatmulReduceScatter(Workload):
         return None
 
 
+class CopyCalibration(Workload):
+    """A plain device-to-device copy of known size: what the HBM byte counters read for it scales the
+    counters of the real kernels (profiles/ states the factors)."""
+
+    bound = "hbm"
+    dtype = "u8"
+
+    def __init__(self, name, nbytes):
+        self.name, self.nbytes, self.flops = name, nbytes, 0
+
+    def algorithmic_bytes(self, world):
+        return 2 * self.nbytes
+
+    def describe(self, world):
+        return {"workload": self.name, "op": "copy", "bytes": self.nbytes}
+
+    def setup(self, iris, world):
+        self.ctx = iris.iris(1 << 20, num_ranks=1, rank=0)
+        self.src = torch.empty(self.nbytes // 4, dtype=torch.int32, device="cuda").fill_(1)
+        self.dst = torch.empty_like(self.src)
+        torch.cuda.synchronize()
+
+    def step(self):
+        self.dst.copy_(self.src)
+
+    def cpu_baseline(self, world, budget_s=20.0):
+        return None
+
+
 WORKLOADS = {
+    "copy_calibration_1GiB": lambda: CopyCalibration("copy_calibration_1GiB", 1 << 30),
     "matmul_all_reduce_bf16_4096x4096x1376": lambda: MatmulAllReduce("matmul_all_reduce_bf16_4096x4096x1376", 4096, 4096, 1376),
     "matmul_all_reduce_two_shot_bf16_4096x4096x1376": lambda: MatmulAllReduce(
         "matmul_all_reduce_two_shot_bf16_4096x4096x1376", 4096, 4096, 1376, variant="two_shot"),
@@ -264,7 +294,7 @@ def main():
     wl = WORKLOADS[args.workload]()
     wl.setup(iris, args.world)
     wall, per_launch_ms = timed_steps(wl, args.steps, args.warmup)
-    kernel = _lib.last_kernel()
+    kernel = _lib.last_kernel() if not isinstance(wl, CopyCalibration) else "torch copy kernel"
     ms_per_step = wall * 1e3 / args.steps
     launch_ms = statistics.mean(per_launch_ms)
     tflops = wl.flops * args.steps / wall / 1e12
@@ -295,7 +325,7 @@ def main():
         "dtype": wl.dtype,
         "data": "synthetic",
         "config": wl.describe(args.world),
-        "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2),
+        "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2) if wl.dtype in PEAK else None,
         "roofline": roofline,
     }
 

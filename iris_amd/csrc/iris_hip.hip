@@ -476,36 +476,52 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     // Loader position: next K step to issue = (i_src, i_kb), i_step overall.
     int i_step = 0, i_src = 0, i_kb = 0;
 
-    // Issue the direct-to-LDS loads of the next K step into ring slot `slot`.  Steps past the end
-    // load nothing (every lane is out of range and deposits zeros), which keeps the per-thread
-    // count of outstanding loads identical on every step.
-    auto issue = [&](int slot) {
+    // The direct-to-LDS loads of one K step, issued one at a time so that the main loop can spread
+    // them between its MFMAs (a wave issues in order: a burst of loads right after the barrier would
+    // hold back the MFMAs behind it while the memory pipeline absorbs the burst).  Steps past the end
+    // load nothing (every lane is out of range and deposits zeros), which keeps the per-thread count
+    // of outstanding loads identical on every step.
+    struct StepLoads {
+      int klim;
+      unsigned sa, sb, a_soff, b_soff;
+    };
+    auto begin_step = [&](int slot) {
+      StepLoads L;
       const bool live = i_step < nsteps;
       const int k0 = i_kb * BK;
-      const int klim = live ? klocal - k0 : 0;  // k elements of this step that exist
-      const unsigned sa = smem_base + slot * CFG::STAGE_BYTES + wave * kDmaBytes;
-      const unsigned sb = sa + CFG::A_BYTES;
-      const unsigned a_soff = (unsigned)(k0 * ES);
+      L.klim = live ? klocal - k0 : 0;  // k elements of this step that exist
+      L.sa = smem_base + slot * CFG::STAGE_BYTES + wave * kDmaBytes;
+      L.sb = L.sa + CFG::A_BYTES;
+      L.a_soff = (unsigned)(k0 * ES);
       const long long kglob = (long long)i_src * klocal + k0;
-#pragma unroll
-      for (int i = 0; i < LA; ++i) {
-        const unsigned v = (la_k[i] < klim) ? a_voff[i] : kInvalidOffset;
-        dma16(ra, sa + i * NW * kDmaBytes, v, a_soff);
-      }
-      const unsigned b_soff = __builtin_amdgcn_readfirstlane(
+      L.b_soff = __builtin_amdgcn_readfirstlane(
           CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
-#pragma unroll
-      for (int i = 0; i < LB; ++i) {
+      return L;
+    };
+    auto issue_one = [&](const StepLoads& L, int j) {  // j in [0, LA + LB)
+      if (j < LA) {
+        const unsigned v = (la_k[j] < L.klim) ? a_voff[j] : kInvalidOffset;
+        dma16(ra, L.sa + j * NW * kDmaBytes, v, L.a_soff);
+      } else {
+        const int i = j - LA;
         const int kpos = CFG::B_KCONTIG ? lb_col[i] : lb_row[i];
-        const unsigned v = (kpos < klim) ? b_voff[i] : kInvalidOffset;
-        dma16(rb, sb + i * NW * kDmaBytes, v, b_soff);
+        const unsigned v = (kpos < L.klim) ? b_voff[i] : kInvalidOffset;
+        dma16(rb, L.sb + i * NW * kDmaBytes, v, L.b_soff);
       }
+    };
+    auto end_step = [&]() {
       ++i_step;
       if (++i_kb == nkb) {  // next source slot (gather along K only)
         i_kb = 0;
         ++i_src;
         if (p.gather == GATHER_K && i_src < nsrc) ra = make_rsrc_words(in_slot(a_own, i_src) + a_tile_off);
       }
+    };
+    auto issue = [&](int slot) {
+      const StepLoads L = begin_step(slot);
+#pragma unroll
+      for (int j = 0; j < LA + LB; ++j) issue_one(L, j);
+      end_step();
     };
 
     MfmaAcc<CFG> acc;
@@ -534,12 +550,12 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       // the fragment reads in flight) orders the operand ring between the waves.
       wait_vmcnt<(STAGES - 3) * (LA + LB)>();  // this thread's loads of step s+1 have landed
       __builtin_amdgcn_s_barrier();             // everyone's have; everyone is past step s-1
-      {
-        int pslot = slot + STAGES - 1;
-        if (pslot >= STAGES) pslot -= STAGES;
-        issue(pslot);                           // refill the slot step s-1 used
-      }
+      int pslot = slot + STAGES - 1;
+      if (pslot >= STAGES) pslot -= STAGES;
+      const StepLoads L = begin_step(pslot);  // refills the slot step s-1 used
       const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
+      constexpr int NSLOT = KS * MB;          // MFMA groups of a step; the loads are spread over them
+      constexpr int NLOAD = LA + LB;
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk) {
         if (kk + 1 < KS)
@@ -548,10 +564,16 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
           load_frags(fr[(kk + 1) & 1], nslot, 0);
         const Frags<CFG>& f = fr[kk & 1];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+          for (int j = 0; j < NLOAD; ++j)
+            if (j * NSLOT / NLOAD == kk * MB + mb) issue_one(L, j);
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(f.a[mb], f.b[nb], acc.v[mb][nb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+      end_step();
       static_assert(KS % 2 == 0 || KS == 1, "fragment double buffer assumes an even slice count");
       if constexpr (KS == 1) {
         // With one slice per step the two buffers alternate across steps.
@@ -623,7 +645,9 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     if (p.epi != EPI_STORE) {
       // Publish: every wave waits until its aux stores have reached L2, the workgroup meets, and
       // the threads that raise flags do so with system-scope release (one L2 write-back per
-      // workgroup instead of one per wave).
+      // workgroup instead of one per wave).  Likewise the peers' flags are polled (system-scope
+      // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
+      // every wave poll and run ahead measured slower.
       wait_vmcnt<0>();
       __syncthreads();
       raise_flags<BM, BN, NT>(p, m0, n0, tid);
@@ -661,8 +685,11 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
 #pragma unroll
           for (int g = 0; g < G; ++g) {
             const int gm = m0 + (pg + g) * RPP + t_row;
-            const int t = (gm / p.flag_bm) * ftn + fcol;
-            owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+            owner[g] = p.rank;
+            if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
+              const int t = (gm / p.flag_bm) * ftn + fcol;
+              owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+            }
             active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
             eoff[g] = active[g] ? ((long long)gm * p.s_cm + gn) * 2 : safe_off;
             if constexpr (NP > 0) {
