@@ -131,16 +131,17 @@ class MatmulAllReduce(Workload):
 class AllGatherMatmul(Workload):
     bound = "bf16"
 
-    def __init__(self, name, M, N, K):
+    def __init__(self, name, M, N, K, b_transposed=False):
         self.name, self.M, self.N, self.K = name, M, N, K
         self.flops = 2 * M * N * K
+        self.b_transposed = b_transposed  # B handed over as the transpose of an (N, K) tensor
 
     def algorithmic_bytes(self, world):
         return 2 * (self.M * self.K + self.K * self.N + self.M * self.N)
 
     def describe(self, world):
         return {"workload": self.name, "op": "all_gather_matmul", "gather": "rows", "M": self.M, "N": self.N,
-                "K": self.K, "W": world}
+                "K": self.K, "W": world, "B_layout": "K-contiguous" if self.b_transposed else "N-contiguous"}
 
     def setup(self, iris, world):
         from iris_amd import ops
@@ -149,8 +150,13 @@ class AllGatherMatmul(Workload):
         self.A = ctx.zeros((M // world, K), dtype=torch.bfloat16)
         for r in range(world):
             ctx.peer_view(self.A, r).copy_(_randn((M // world, K), r, torch.bfloat16, K ** -0.5))
-        self.B = ctx.zeros((K, N), dtype=torch.bfloat16)
-        self.B.copy_(_randn((K, N), 8, torch.bfloat16, K ** -0.5))
+        if self.b_transposed:
+            self.B = ctx.zeros((N, K), dtype=torch.bfloat16)
+            self.B.copy_(_randn((K, N), 8, torch.bfloat16, K ** -0.5).t())
+            self.B = self.B.t()
+        else:
+            self.B = ctx.zeros((K, N), dtype=torch.bfloat16)
+            self.B.copy_(_randn((K, N), 8, torch.bfloat16, K ** -0.5))
         self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
         self._op = ops.all_gather_matmul
         torch.cuda.synchronize()
@@ -244,6 +250,7 @@ WORKLOADS = {
     "matmul_all_reduce_two_shot_bf16_4096x4096x1376": lambda: MatmulAllReduce(
         "matmul_all_reduce_two_shot_bf16_4096x4096x1376", 4096, 4096, 1376, variant="two_shot"),
     "all_gather_matmul_bf16_8192x1792x4096": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096", 8192, 1792, 4096),
+    "all_gather_matmul_bf16_8192x1792x4096_nt": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096_nt", 8192, 1792, 4096, b_transposed=True),
     "matmul_reduce_scatter_bf16_8192x4096x1376": lambda: MatmulReduceScatter("matmul_reduce_scatter_bf16_8192x4096x1376", 8192, 4096, 1376),
     "matmul_all_reduce_fp8_16384x8192x1024": lambda: MatmulAllReduce("matmul_all_reduce_fp8_16384x8192x1024", 16384, 8192, 1024, fp8=True),
     "matmul_all_reduce_fp8_skinny_32x8192x1024": lambda: MatmulAllReduce(

@@ -631,14 +631,34 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     const bool col_ok = gn < p.N;
     const char* const t_lds = smem + t_row * CFG::TROW + t_chunk * 16;
 
-    // Phase 1: C (plain store) or aux (own slot).
+    // Phase 1: C (plain store) or aux (own slot).  When no peer contributes (world of one, or peers
+    // switched off) the reduced tile equals the own tile, so C is written in the same pass and
+    // phase 2 is skipped.
+    const bool solo = (p.epi != EPI_STORE) && (!p.sum_peers || p.world == 1);
     {
       char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+      const int ftn1 = cdiv(p.N, p.flag_bn);
+      const int ftotal1 = cdiv(p.M, p.flag_bm) * ftn1;
 #pragma unroll 4
       for (int ps = 0; ps < PASSES; ++ps) {
         const int gm = m0 + ps * RPP + t_row;
         const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + ps * RPP * CFG::TROW);
-        if (gm < p.M && col_ok) *(u32x4_t*)(out1 + ((long long)gm * p.s_cm + gn) * 2) = v;
+        if (gm < p.M && col_ok) {
+          const long long eoff = ((long long)gm * p.s_cm + gn) * 2;
+          *(u32x4_t*)(out1 + eoff) = v;
+          if (solo) {
+            int owner = p.rank;
+            if (p.epi != EPI_ONE_SHOT) owner = owner_of(p.epi, (gm / p.flag_bm) * ftn1 + gn / p.flag_bn, ftotal1, p.world, p.rank);
+            if (p.all_owners || owner == p.rank) {
+              if (p.epi == EPI_TWO_SHOT) {
+                for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot((unsigned long long)p.C, pr) + eoff) = v;
+              } else {
+                const int dst = p.all_owners ? owner : p.rank;
+                *(u32x4_t*)(in_slot((unsigned long long)p.C, dst) + eoff) = v;
+              }
+            }
+          }
+        }
       }
     }
 
@@ -651,7 +671,7 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       wait_vmcnt<0>();
       __syncthreads();
       raise_flags<BM, BN, NT>(p, m0, n0, tid);
-      if (p.sum_peers && p.world > 1) {
+      if (!solo) {
         wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
         __syncthreads();
       }
@@ -741,8 +761,8 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
           }
         }
       };
-      switch (p.world <= kMaxCachedSlots ? npeers : -1) {
-        case 0: reduce_tile(std::integral_constant<int, 0>{}); break;
+      switch (solo ? -2 : (p.world <= kMaxCachedSlots ? npeers : -1)) {
+        case -2: break;  // C was written in phase 1
         case 1: reduce_tile(std::integral_constant<int, 1>{}); break;
         case 3: reduce_tile(std::integral_constant<int, 3>{}); break;
         case 7: reduce_tile(std::integral_constant<int, 7>{}); break;
