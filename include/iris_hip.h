@@ -36,8 +36,10 @@ enum {
   IRIS_HIP_FP8_E4M3 = 3 /* OCP e4m3fn, inputs only; products are multiplied by `scale` */
 };
 
-/* All-reduce variants (the strings of FusedConfig.all_reduce_variant, iris/ops/config.py:62). */
+/* All-reduce variants (the strings of FusedConfig.all_reduce_variant, iris/ops/config.py:62), numbered
+ * like AllReduceConfig.variant_code (iris/mem/triton/types.py:285-292). */
 enum {
+  IRIS_HIP_VARIANT_ATOMIC = 0,   /* iris/mem/triton/context.py:689-702 */
   IRIS_HIP_VARIANT_ONE_SHOT = 2, /* iris/mem/triton/context.py:733-764 */
   IRIS_HIP_VARIANT_TWO_SHOT = 3  /* iris/mem/triton/context.py:801-839 */
 };
@@ -70,7 +72,9 @@ enum {
 /*
  * Fused C = all_reduce(A @ B), rank-local part.
  * Replaces the launch of _fused_matmul_all_reduce_kernel
- * (iris/ops/matmul_all_reduce.py:334-362; kernel :25-145) for VARIANT one_shot / two_shot.
+ * (iris/ops/matmul_all_reduce.py:334-362; kernel :25-145) for VARIANT atomic / one_shot / two_shot.
+ *
+ * atomic: cast(A @ B) is added atomically into C of every slot (aux_buffer and locks may be NULL).
  *
  * Per flag tile t = pid_m * cdiv(N, block_size_n) + pid_n of block_size_m x block_size_n elements:
  *   aux[tile]   = cast(A @ B)              (own slot)
@@ -144,6 +148,24 @@ int iris_hip_all_gather_matmul(const void* A_sharded, const void* B, void* C, co
                                const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
                                int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
                                int32_t gather_dim,
+                               int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype, float scale,
+                               int32_t path, void* stream);
+
+/*
+ * Fused C_gathered = all_gather(A @ B (+ bias[:, None])) along rows, rank-local part (scatter pattern).
+ * Replaces the launch of _fused_matmul_all_gather_kernel (iris/ops/matmul_all_gather.py:27-105, launch
+ * :222-262; DeviceContext.all_gather iris/mem/triton/context.py:841-864).
+ *
+ * A is M_local x K; the product tile is cast and stored into rows [cur_rank*M_local, (cur_rank+1)*M_local)
+ * of C_gathered (M x N, M = M_local * world_size) in EVERY slot.  bias (may be NULL) has M_local elements.
+ */
+int iris_hip_matmul_all_gather(const void* A, const void* B, void* C_gathered, const void* bias,
+                               int64_t M_local, int64_t M, int64_t N, int64_t K,
+                               int64_t stride_am, int64_t stride_ak,
+                               int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm_gathered, int64_t stride_cn_gathered, int64_t stride_bias,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
                                int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype, float scale,
                                int32_t path, void* stream);
 

@@ -11,11 +11,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # IRIS_HIP_LIBRARY names another build of the same library (e.g. one compiled with other tile shapes).
 LIBRARY_PATH = os.environ.get("IRIS_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libiris_hip.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # Enumerations of include/iris_hip.h
 BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
-VARIANT_ONE_SHOT, VARIANT_TWO_SHOT = 2, 3
+VARIANT_ATOMIC, VARIANT_ONE_SHOT, VARIANT_TWO_SHOT = 0, 2, 3
 ACC_FP32, ACC_REFERENCE = 0, 1
 GATHER_K, GATHER_M = 1, 2
 PATH_AUTO, PATH_MFMA, PATH_GENERIC = 0, 1, 2
@@ -50,6 +50,16 @@ PROTOTYPES = {
          _ptr, _i32, _i32,  # context_tensor, cur_rank, world_size
          _i32, _i32, _i32,  # block sizes
          _i32,  # gather_dim
+         _i32, _i32, _i32, _f32,  # in_dtype, out_dtype, bias_dtype, scale
+         _i32, _ptr],  # path, stream
+    ),
+    "iris_hip_matmul_all_gather": (
+        _i32,
+        [_ptr, _ptr, _ptr, _ptr,  # A, B, C_gathered, bias
+         _i64, _i64, _i64, _i64,  # M_local, M, N, K
+         _i64, _i64, _i64, _i64, _i64, _i64, _i64,  # strides am ak bk bn cm cn bias
+         _ptr, _i32, _i32,  # context_tensor, cur_rank, world_size
+         _i32, _i32, _i32,  # block sizes
          _i32, _i32, _i32, _f32,  # in_dtype, out_dtype, bias_dtype, scale
          _i32, _ptr],  # path, stream
     ),

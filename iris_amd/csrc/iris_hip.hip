@@ -45,7 +45,10 @@ typedef __attribute__((ext_vector_type(4))) short i16x4_t;
 typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
 typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 
-enum { EPI_STORE = 0, EPI_ONE_SHOT = 1, EPI_TWO_SHOT = 2, EPI_REDUCE_SCATTER = 3 };
+enum { EPI_STORE = 0, EPI_ONE_SHOT = 1, EPI_TWO_SHOT = 2, EPI_REDUCE_SCATTER = 3, EPI_ALL_GATHER = 4, EPI_ATOMIC = 5 };
+
+// Epilogues that publish aux + flags and then reduce over the slots.
+__host__ __device__ inline bool epi_has_flags(int epi) { return epi == EPI_ONE_SHOT || epi == EPI_TWO_SHOT || epi == EPI_REDUCE_SCATTER; }
 enum { GATHER_NONE = 0, GATHER_K = 1, GATHER_M = 2 };
 
 struct FusedParams {
@@ -72,6 +75,7 @@ struct FusedParams {
   long long spin_limit;
   int* status;
   int tiles_m, tiles_n, group_m, num_xcd;
+  int row_offset;  // all-gather: first row of this rank's block in the gathered output
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -109,6 +113,19 @@ struct OutF16 {
   static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_f16_bits(f); }
   static constexpr bool kFp32SumInReference = true;
 };
+
+// Atomically add two packed 16-bit floats (one 32-bit word) to memory.
+typedef __attribute__((ext_vector_type(2))) short s16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <class Out>
+__device__ __forceinline__ void atomic_add_packed(char* addr, unsigned word) {
+  if constexpr (Out::kFp32SumInReference)  // float16
+    __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) f16x2_t*)addr,
+                                              __builtin_bit_cast(f16x2_t, word));
+  else
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) s16x2_t*)addr,
+                                               __builtin_bit_cast(s16x2_t, word));
+}
 
 __device__ __forceinline__ float load_scalar_as_float(const char* base, long long idx, int dtype) {
   if (dtype == IRIS_HIP_FP32) return ((const float*)base)[idx];
@@ -634,27 +651,41 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     // Phase 1: C (plain store) or aux (own slot).  When no peer contributes (world of one, or peers
     // switched off) the reduced tile equals the own tile, so C is written in the same pass and
     // phase 2 is skipped.
-    const bool solo = (p.epi != EPI_STORE) && (!p.sum_peers || p.world == 1);
+    const bool flags = epi_has_flags(p.epi);
+    const bool solo = flags && (!p.sum_peers || p.world == 1);
     {
-      char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+      char* const out1 = flags ? p.aux : p.C;
       const int ftn1 = cdiv(p.N, p.flag_bn);
       const int ftotal1 = cdiv(p.M, p.flag_bm) * ftn1;
+      const unsigned long long c_base = (unsigned long long)p.C;
 #pragma unroll 4
       for (int ps = 0; ps < PASSES; ++ps) {
         const int gm = m0 + ps * RPP + t_row;
         const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + ps * RPP * CFG::TROW);
         if (gm < p.M && col_ok) {
-          const long long eoff = ((long long)gm * p.s_cm + gn) * 2;
-          *(u32x4_t*)(out1 + eoff) = v;
+          const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gn) * 2;
+          if (p.epi == EPI_ALL_GATHER) {
+            // the tile goes to every rank's gathered output (iris/mem/triton/context.py:841-864)
+            for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
+          } else if (p.epi == EPI_ATOMIC) {
+            // the tile is added into every rank's C (iris/mem/triton/context.py:689-702)
+            for (int pr = 0; pr < p.world; ++pr) {
+              char* dst = (char*)(in_slot(c_base, pr) + eoff);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) atomic_add_packed<Out>(dst + 4 * e, v[e]);
+            }
+          } else {
+            *(u32x4_t*)(out1 + eoff) = v;
+          }
           if (solo) {
             int owner = p.rank;
             if (p.epi != EPI_ONE_SHOT) owner = owner_of(p.epi, (gm / p.flag_bm) * ftn1 + gn / p.flag_bn, ftotal1, p.world, p.rank);
             if (p.all_owners || owner == p.rank) {
               if (p.epi == EPI_TWO_SHOT) {
-                for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot((unsigned long long)p.C, pr) + eoff) = v;
+                for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
               } else {
                 const int dst = p.all_owners ? owner : p.rank;
-                *(u32x4_t*)(in_slot((unsigned long long)p.C, dst) + eoff) = v;
+                *(u32x4_t*)(in_slot(c_base, dst) + eoff) = v;
               }
             }
           }
@@ -662,7 +693,7 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       }
     }
 
-    if (p.epi != EPI_STORE) {
+    if (flags) {
       // Publish: every wave waits until its aux stores have reached L2, the workgroup meets, and
       // the threads that raise flags do so with system-scope release (one L2 write-back per
       // workgroup instead of one per wave).  Likewise the peers' flags are polled (system-scope
@@ -777,11 +808,29 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
 // ------------------------------------------------------------------------------------------------
 // Generic kernel: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMA.
 // ------------------------------------------------------------------------------------------------
+// Atomic add of one 16-bit float: compare-and-swap on the aligned 32-bit word that contains it.
+template <class E>
+__device__ __forceinline__ void atomic_add_half(char* p, float f) {
+  unsigned* word = (unsigned*)((unsigned long long)p & ~3ull);
+  const int shift = ((unsigned long long)p & 2) ? 16 : 0;
+  unsigned old = *word, assumed;
+  do {
+    assumed = old;
+    unsigned short cur = (unsigned short)(assumed >> shift);
+    float sum = E::load((const char*)&cur) + f;
+    unsigned short nv;
+    E::store((char*)&nv, sum);
+    const unsigned repl = (assumed & ~(0xFFFFu << shift)) | ((unsigned)nv << shift);
+    old = atomicCAS(word, assumed, repl);
+  } while (old != assumed);
+}
+
 struct ElemBF16 {
   static constexpr int size = 2;
   static __device__ __forceinline__ float load(const char* p) { return bf16_bits_to_float(*(const unsigned short*)p); }
   static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_bf16_bits(f); }
   static __device__ __forceinline__ float round(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
+  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomic_add_half<ElemBF16>(p, f); }
   static constexpr bool kFp32SumInReference = false;
 };
 struct ElemF16 {
@@ -789,6 +838,7 @@ struct ElemF16 {
   static __device__ __forceinline__ float load(const char* p) { return f16_bits_to_float(*(const unsigned short*)p); }
   static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_f16_bits(f); }
   static __device__ __forceinline__ float round(float f) { return f16_bits_to_float(float_to_f16_bits(f)); }
+  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomic_add_half<ElemF16>(p, f); }
   static constexpr bool kFp32SumInReference = true;
 };
 struct ElemF32 {
@@ -796,6 +846,7 @@ struct ElemF32 {
   static __device__ __forceinline__ float load(const char* p) { return *(const float*)p; }
   static __device__ __forceinline__ void store(char* p, float f) { *(float*)p = f; }
   static __device__ __forceinline__ float round(float f) { return f; }
+  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomicAdd((float*)p, f); }
   static constexpr bool kFp32SumInReference = false;  // fp32 data sums in fp32 either way
 };
 struct ElemFP8 {
@@ -887,15 +938,24 @@ __global__ void __launch_bounds__(256) fused_generic_kernel(const FusedParams p)
 #pragma unroll
       for (int j = 0; j < 4; ++j) own[i][j] = Out::round(acc[i][j] * p.scale + badd);
     }
-    char* const out1 = (p.epi == EPI_STORE) ? p.C : p.aux;
+    const bool flags = epi_has_flags(p.epi);
+    char* const out1 = flags ? p.aux : p.C;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int gm = m0 + ty * 4 + i, gn = n0 + tx * 4 + j;
-        if (gm < p.M && gn < p.N) Out::store(out1 + ((long long)gm * p.s_cm + (long long)gn * p.s_cn) * Out::size, own[i][j]);
+        if (!(gm < p.M && gn < p.N)) continue;
+        const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + (long long)gn * p.s_cn) * Out::size;
+        if (p.epi == EPI_ALL_GATHER) {
+          for (int pr = 0; pr < p.world; ++pr) Out::store(slot_ptr(p.heap_bases, p.C, p.rank, pr) + eoff, own[i][j]);
+        } else if (p.epi == EPI_ATOMIC) {
+          for (int pr = 0; pr < p.world; ++pr) Out::atomic_add(slot_ptr(p.heap_bases, p.C, p.rank, pr) + eoff, own[i][j]);
+        } else {
+          Out::store(out1 + eoff, own[i][j]);
+        }
       }
-    if (p.epi == EPI_STORE) continue;
+    if (!flags) continue;
 
     __atomic_thread_fence(__ATOMIC_RELEASE);
     __syncthreads();
@@ -1094,7 +1154,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("M, N, K must be positive (got %d, %d, %d)", p.M, p.N, p.K);
   if (!p.A || !p.B || !p.C) return fail("A, B and C must not be NULL");
   if (p.world < 1 || p.rank < 0 || p.rank >= p.world) return fail("bad rank/world_size %d/%d", p.rank, p.world);
-  if (p.epi != EPI_STORE) {
+  if (epi_has_flags(p.epi)) {
     if (!p.aux || !p.locks) return fail("aux_buffer and locks must not be NULL");
     if (p.flag_bm <= 0 || p.flag_bn <= 0) return fail("block sizes must be positive");
   } else {
@@ -1148,8 +1208,8 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
                                void* stream) {
   (void)block_size_k;
   if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
-  if (variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
-    return fail("variant %d is not one_shot (2) or two_shot (3)", variant);
+  if (variant != IRIS_HIP_VARIANT_ATOMIC && variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
+    return fail("variant %d is not atomic (0), one_shot (2) or two_shot (3)", variant);
   FusedParams p;
   memset(&p, 0, sizeof(p));
   p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C; p.aux = (char*)aux_buffer; p.locks = locks;
@@ -1159,7 +1219,7 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
   p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
   p.rank = cur_rank; p.world = world_size;
   p.flag_bm = block_size_m; p.flag_bn = block_size_n;
-  p.epi = variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
+  p.epi = variant == IRIS_HIP_VARIANT_ATOMIC ? EPI_ATOMIC : variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
   p.acc_mode = acc_mode; p.all_owners = 0; p.sum_peers = 1;
   p.scale = scale; p.spin_limit = spin_limit; p.status = status;
   return run_fused(p, in_dtype, out_dtype, path, stream);
@@ -1226,6 +1286,33 @@ int iris_hip_all_gather_matmul(const void* A_sharded, const void* B, void* C, co
   return run_fused(p, in_dtype, out_dtype, path, stream);
 }
 
+int iris_hip_matmul_all_gather(const void* A, const void* B, void* C_gathered, const void* bias,
+                               int64_t M_local, int64_t M, int64_t N, int64_t K,
+                               int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm_gathered, int64_t stride_cn_gathered, int64_t stride_bias,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype, float scale,
+                               int32_t path, void* stream) {
+  (void)block_size_m; (void)block_size_n; (void)block_size_k;
+  if (!fits_int(M_local) || !fits_int(M) || !fits_int(N) || !fits_int(K))
+    return fail("M_local, M, N, K must be in [1, 2^31)");
+  if (world_size < 1 || M != M_local * world_size)
+    return fail("M (%lld) must equal M_local (%lld) * world_size (%d)", (long long)M, (long long)M_local, world_size);
+  if (bias && elem_size(bias_dtype) < 2) return fail("unsupported bias type %d", bias_dtype);
+  FusedParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C_gathered; p.bias = (const char*)bias;
+  p.M = (int)M_local; p.N = (int)N; p.K = (int)K; p.K_local = (int)K; p.gather = GATHER_NONE;
+  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
+  p.s_cm = stride_cm_gathered; p.s_cn = stride_cn_gathered; p.s_bias = stride_bias; p.bias_dtype = bias_dtype;
+  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
+  p.rank = cur_rank; p.world = world_size;
+  p.row_offset = (int)(cur_rank * M_local);
+  p.epi = EPI_ALL_GATHER; p.scale = scale;
+  return run_fused(p, in_dtype, out_dtype, path, stream);
+}
+
 int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_t* lds_bytes_per_block) {
   g_last_error[0] = 0;
   DeviceFacts* f = nullptr;
@@ -1239,6 +1326,6 @@ int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }
-int iris_hip_abi_version(void) { return 1; }
+int iris_hip_abi_version(void) { return 2; }
 
 }  // extern "C"

@@ -5,12 +5,13 @@
     shmem.ops.matmul_all_reduce(C, A, B)          # via the context
     iris.ops.matmul_all_reduce(shmem, C, A, B)    # or as free functions
 
-Mirrors iris/ops/__init__.py:43-186 of the reference for matmul_all_reduce, all_gather_matmul and
-matmul_reduce_scatter.
+Mirrors iris/ops/__init__.py:43-186 of the reference: matmul_all_reduce, all_gather_matmul,
+matmul_all_gather and matmul_reduce_scatter.
 """
 
 from .all_gather_matmul import all_gather_matmul, all_gather_matmul_preamble
 from .config import FusedConfig
+from .matmul_all_gather import matmul_all_gather, matmul_all_gather_preamble
 from .matmul_all_reduce import matmul_all_reduce, matmul_all_reduce_preamble
 from .matmul_reduce_scatter import matmul_reduce_scatter, matmul_reduce_scatter_preamble
 from .workspace import FusedWorkspace
@@ -33,6 +34,11 @@ class OpsNamespace:
         return all_gather_matmul(self._shmem, output_tensor, A_sharded, B, bias, async_op, config, workspace,
                                  **kwargs)
 
+    def matmul_all_gather(self, output_tensor, A, B, bias=None, async_op=False, config=None, workspace=None,
+                          **kwargs):
+        """output = all_gather(A @ B + bias[:, None]) along rows."""
+        return matmul_all_gather(self._shmem, output_tensor, A, B, bias, async_op, config, workspace, **kwargs)
+
     def matmul_reduce_scatter(self, output_tensor, A, B, bias=None, async_op=False, config=None, workspace=None,
                               **kwargs):
         """output = reduce_scatter(A @ B).  `bias` is accepted and ignored.  (The reference forwards
@@ -48,6 +54,8 @@ __all__ = [
     "matmul_all_reduce_preamble",
     "all_gather_matmul",
     "all_gather_matmul_preamble",
+    "matmul_all_gather",
+    "matmul_all_gather_preamble",
     "matmul_reduce_scatter",
     "matmul_reduce_scatter_preamble",
 ]

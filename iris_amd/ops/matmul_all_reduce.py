@@ -17,7 +17,7 @@ from ._common import (acc_code, current_stream, dtype_code, iris_launch, is_fp8,
 from .config import FusedConfig
 from .workspace import FusedWorkspace
 
-_VARIANT_CODES = {"one_shot": _lib.VARIANT_ONE_SHOT, "two_shot": _lib.VARIANT_TWO_SHOT}
+_VARIANT_CODES = {"atomic": _lib.VARIANT_ATOMIC, "one_shot": _lib.VARIANT_ONE_SHOT, "two_shot": _lib.VARIANT_TWO_SHOT}
 
 
 def _tile_count(M, N, config):
@@ -92,7 +92,8 @@ def matmul_all_reduce(
     """C = all_reduce(A @ B) for this rank; returns the workspace (reusable on the next call).
 
     A is (M, K), different on every rank; B is (K, N), replicated; C is (M, N).  With variant
-    "one_shot" this rank sums every tile of its own product with the peers' tiles (read from their
+    "atomic" the rank's product is added atomically into every rank's C (which the preamble zeroed);
+    with "one_shot" this rank sums every tile of its own product with the peers' tiles (read from their
     aux buffers once their flags are up) into its own C; with "two_shot" it does so only for the
     tiles t with t % world_size == rank and writes the result into every rank's C.
 
@@ -135,7 +136,7 @@ def matmul_all_reduce(
     if config.all_reduce_variant not in _VARIANT_CODES:
         config.validate(world_size=world_size)
         raise NotImplementedError(
-            f"all_reduce_variant {config.all_reduce_variant!r} has no HIP kernel; use 'one_shot' or 'two_shot'"
+            f"all_reduce_variant {config.all_reduce_variant!r} has no HIP kernel; use 'atomic', 'one_shot' or 'two_shot'"
         )
     needs_prepare = workspace is None or not workspace.matches(
         "matmul_all_reduce", (M, N, K), A.dtype, world_size, config.all_reduce_variant
@@ -151,13 +152,17 @@ def matmul_all_reduce(
             f"Lock array too small: have {workspace.locks.numel()} but need {total_tiles}. "
             f"Pre-allocate workspace with the smallest block sizes you intend to use."
         )
-    if workspace.aux_buffer is None or workspace.locks is None:
-        raise ValueError("workspace has no aux buffer / locks for the one_shot / two_shot variants")
-    if workspace.aux_buffer.dtype != C.dtype:
-        raise ValueError(f"workspace aux buffer has dtype {workspace.aux_buffer.dtype}, C has {C.dtype}")
-    # aux is addressed with C's strides, as in the reference kernel.
-    if (M - 1) * stride_cm + (N - 1) * stride_cn >= workspace.aux_buffer.numel():
-        raise ValueError("C's strides address beyond the aux buffer")
+    if config.all_reduce_variant == "atomic":
+        if not shmem.is_symmetric(C):
+            raise RuntimeError("C must be allocated on the symmetric heap (every rank's copy is added to)")
+    else:
+        if workspace.aux_buffer is None or workspace.locks is None:
+            raise ValueError("workspace has no aux buffer / locks for the one_shot / two_shot variants")
+        if workspace.aux_buffer.dtype != C.dtype:
+            raise ValueError(f"workspace aux buffer has dtype {workspace.aux_buffer.dtype}, C has {C.dtype}")
+        # aux is addressed with C's strides, as in the reference kernel.
+        if (M - 1) * stride_cm + (N - 1) * stride_cn >= workspace.aux_buffer.numel():
+            raise ValueError("C's strides address beyond the aux buffer")
 
     scale = 1.0
     if is_fp8(A.dtype):

@@ -25,7 +25,7 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
                                                  a KAT that separates the fp32 rule from the reference's
                                                  data-type rule
   matmul_all_reduce / matmul_reduce_scatter /
-  all_gather_matmul                             pinned: W=1 reduces to gemm; closed-form peers; the
+  all_gather_matmul / matmul_all_gather         pinned: W=1 reduces to gemm; closed-form peers; the
                                                  reference tests' checks (torch.cat(shards, 1) @ B,
                                                  tests/ops/test_all_gather_matmul.py:61-66)
   flag contents                                 source-pinned only (no reference test asserts them):
@@ -206,6 +206,14 @@ def matmul_all_reduce(A, B, peer_aux, rank, world, block_m, block_n, variant, mo
     out_dtype = out_dtype or A.dtype
     M, N = A.shape[0], B.shape[1]
     own = gemm(A, B, out_dtype, scale)
+    if variant == "atomic":
+        # iris/mem/triton/context.py:689-702: the own tile is atomically added to C on every rank
+        # (one add in the data type per element).  peer_aux[r], if given, is what C of rank r held before.
+        C = []
+        for r in range(world):
+            before = peer_aux[r] if peer_aux is not None and peer_aux[r] is not None else torch.zeros(M, N, dtype=out_dtype)
+            C.append((before.to(torch.float32) + own.to(torch.float32)).to(out_dtype))
+        return dict(aux=None, locks=None, C=C)
     tiles_m, tiles_n = tile_grid(M, N, block_m, block_n)
     locks = np.ones(tiles_m * tiles_n, dtype=np.int32)
     peers = [peer_aux[r] for r in range(world) if r != rank]
@@ -257,6 +265,25 @@ def all_gather_matmul(shards, B, bias=None, gather_dim=1, out_dtype=None, scale=
     """
     A = torch.cat(list(shards), dim=1 if gather_dim == 1 else 0)
     return gemm(A, B, out_dtype or A.dtype, scale, bias)
+
+
+def matmul_all_gather(A, B, rank, world, bias=None, out_dtype=None, scale=1.0):
+    """What rank `rank` writes: its product block into rows [rank*M_local, (rank+1)*M_local) of the
+    gathered (M, N) output of every rank; rows of other ranks are left alone (returned as zeros).
+
+    iris/ops/matmul_all_gather.py:77-105; iris/mem/triton/context.py:841-864 (dim = 0).  The
+    reference test compares with torch.cat(all_gather(A_r @ B), dim=0)
+    (tests/ops/test_matmul_all_gather.py:59-66).
+    """
+    out_dtype = out_dtype or A.dtype
+    M_local, N = A.shape[0], B.shape[1]
+    block = gemm(A, B, out_dtype, scale, bias)
+    out = []
+    for _ in range(world):
+        full = torch.zeros(M_local * world, N, dtype=out_dtype)
+        full[rank * M_local:(rank + 1) * M_local] = block
+        out.append(full)
+    return out
 
 
 # ----------------------------------------------------------------------------------------------

@@ -286,6 +286,59 @@ def test_all_gather_matmul_random_via_namespace():
 
 
 # ------------------------------------------------------------------------------------------------
+# matmul + all-gather (scatter pattern) and the atomic all-reduce variant
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (512, 256, 512), (1024, 2048, 1024)])
+def test_matmul_all_gather(path, dtype, M, N, K):
+    """Shapes of tests/ops/test_matmul_all_gather.py:18-30 of the reference, W = 4, every rank in turn."""
+    W = 4
+    M_local = M // W
+    if M_local < 16:
+        pytest.skip("M_local too small")
+    B = randint_cpu((K, N), 77, dtype, -2, 3)
+    As = [randint_cpu((M_local, K), 80 + r, dtype, -2, 3) for r in range(W)]
+    bias = randint_cpu((M_local,), 90, dtype, -4, 5)
+    bm = 16 if M_local < 64 else 64
+    cfg = iris.FusedConfig(block_size_m=bm, block_size_n=64, block_size_k=32)
+    for rank in (0, W - 1):
+        ctx = _ctx(W, rank)
+        dA, dB, dbias = heap_tensor(ctx, As[rank]), heap_tensor(ctx, B), heap_tensor(ctx, bias)
+        out = ctx.zeros((M, N), dtype=dtype)
+        for r in range(W):
+            ctx.peer_view(out, r).zero_()
+        ctx.ops.matmul_all_gather(out, dA, dB, bias=dbias, config=cfg, kernel_path=path)
+        assert _lib.last_kernel().startswith(path)
+        exp = oracle.matmul_all_gather(As[rank], B, rank, W, bias=bias)
+        for r, got in enumerate(slot_copies(ctx, out)):
+            assert_bits_equal(got, exp[r], f"{_lib.last_kernel()} rank {rank} slot {r}")
+
+
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_all_reduce_atomic(path, dtype):
+    if dtype == torch.float32 and path == "mfma":
+        pytest.skip("fp32 data runs on the generic kernel")
+    W, rank = 4, 2
+    M, N, K = 256, 192, 64
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 21, dtype), randint_cpu((K, N), 22, dtype)
+    before = [randint_cpu((M, N), 300 + r, dtype, -50, 51) for r in range(W)]  # what C held: the peers' adds so far
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="atomic")
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    assert ws.locks is None and ws.aux_buffer is None
+    for r in range(W):
+        ctx.peer_view(dC, r).copy_(before[r])
+    ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, kernel_path=path)
+    exp = oracle.matmul_all_reduce(A, B, before, rank, W, 64, 64, "atomic")
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert_bits_equal(got, exp["C"][r], f"{_lib.last_kernel()} slot {r}")
+
+
+# ------------------------------------------------------------------------------------------------
 # float8 inputs
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("path", ["mfma", "generic"])

@@ -213,8 +213,11 @@ def test_matmul_all_reduce_argument_errors():
         ops.matmul_all_reduce(ctx, C, A, B, config=iris.FusedConfig(block_size_m=512, block_size_n=64, block_size_k=32))
     with pytest.raises(AssertionError, match="too small for block_size_k"):
         ops.matmul_all_reduce(ctx, C, A, B, config=iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=128))
-    with pytest.raises(NotImplementedError, match="atomic"):
-        ops.matmul_all_reduce(ctx, C, A, B, config=iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="atomic"))
+    with pytest.raises(NotImplementedError, match="ring"):
+        ops.matmul_all_reduce(ctx, C, A, B, config=iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="ring"))
+    atomic = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant="atomic")
+    ws = ops.matmul_all_reduce_preamble(ctx, C, A, B, config=atomic)
+    assert ws.locks is None and ws.aux_buffer is None  # reference: no buffers for the atomic variant
     with pytest.raises(ValueError, match="slot_sum"):
         ops.matmul_all_reduce(ctx, C, A, B, config=cfg, slot_sum="fp64")
     # a well-formed call reaches the launch and is refused there: the heap is host memory
@@ -222,6 +225,26 @@ def test_matmul_all_reduce_argument_errors():
         ops.matmul_all_reduce(ctx, C, A, B, config=cfg)
     with pytest.raises(RuntimeError, match="need a GPU context"):
         ctx.ops.matmul_reduce_scatter(C, A, B, config=cfg)
+
+
+def test_matmul_all_gather_argument_errors():
+    ctx = cpu_ctx(heap=1 << 24, world=4)
+    A = ctx.zeros((64, 32), dtype=torch.float16)
+    B = ctx.zeros((32, 64), dtype=torch.float16)
+    out = ctx.zeros((256, 64), dtype=torch.float16)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32)
+    ws = ops.matmul_all_gather_preamble(ctx, A, B, cfg)
+    assert ws.prepared and ws.shape == (256, 64, 32) and ws.operation == "matmul_all_gather"
+    with pytest.raises(AssertionError, match="Inner dimensions must match"):
+        ops.matmul_all_gather(ctx, out, A, ctx.zeros((16, 64), dtype=torch.float16), config=cfg)
+    with pytest.raises(AssertionError, match="Output must be"):
+        ops.matmul_all_gather(ctx, ctx.zeros((64, 64), dtype=torch.float16), A, B, config=cfg)
+    with pytest.raises(AssertionError, match="M_local"):
+        ops.matmul_all_gather(ctx, out, A, B, config=iris.FusedConfig(block_size_m=128, block_size_n=64, block_size_k=32))
+    with pytest.raises(RuntimeError, match="symmetric heap"):
+        ops.matmul_all_gather(ctx, torch.zeros((256, 64), dtype=torch.float16), A, B, config=cfg)
+    with pytest.raises(RuntimeError, match="need a GPU context"):
+        ctx.ops.matmul_all_gather(out, A, B, config=cfg)
 
 
 def test_all_gather_matmul_argument_errors():

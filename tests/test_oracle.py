@@ -213,3 +213,34 @@ def test_all_gather_matmul_both_layouts():
     rows = oracle.all_gather_matmul(shards, B2, gather_dim=0)
     for r in range(W):
         assert torch.equal(rows[6 * r:6 * r + 6], (shards[r].float() @ B2.float()).half())
+
+
+def test_matmul_all_gather_rows():
+    """torch.cat(all_gather(A_r @ B), dim=0) (tests/ops/test_matmul_all_gather.py:59-66 of the reference)."""
+    W, M_local, K, N = 4, 6, 5, 7
+    As = [randint_cpu((M_local, K), 30 + r, torch.float16) for r in range(W)]
+    B = randint_cpu((K, N), 40, torch.float16)
+    expected = torch.cat([(a.float() @ B.float()).half() for a in As], dim=0)
+    total = [torch.zeros(W * M_local, N, dtype=torch.float16) for _ in range(W)]
+    for rank in range(W):
+        written = oracle.matmul_all_gather(As[rank], B, rank, W)
+        for r in range(W):
+            total[r] += written[r]  # every rank writes a disjoint row block into every rank's output
+    for r in range(W):
+        assert torch.equal(total[r], expected)
+    bias = torch.arange(M_local, dtype=torch.float16)
+    with_bias = oracle.matmul_all_gather(As[2], B, 2, W, bias=bias)[0]
+    assert torch.equal(with_bias[12:18], ((As[2].float() @ B.float()) + bias.float()[:, None]).half())
+    assert torch.all(with_bias[:12] == 0) and torch.all(with_bias[18:] == 0)
+
+
+def test_all_reduce_atomic_variant():
+    """Every rank adds its product into every rank's C: after all ranks, C = sum of the products."""
+    W, M, N, K = 4, 8, 8, 8
+    As = [randint_cpu((M, K), 50 + r, torch.float32) for r in range(W)]
+    B = randint_cpu((K, N), 60, torch.float32)
+    C = [torch.zeros(M, N) for _ in range(W)]
+    for rank in range(W):
+        C = oracle.matmul_all_reduce(As[rank], B, C, rank, W, 4, 4, "atomic")["C"]
+    for r in range(W):
+        assert torch.equal(C[r], sum(a @ B for a in As))
