@@ -259,6 +259,16 @@ WORKLOADS = {
 DEFAULT = "matmul_all_reduce_bf16_4096x4096x1376"
 
 
+def measured_traffic(workload, world):
+    """HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs recorded under profiles/
+    (taken with the default W = 8); None when no profile covers this workload."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if world != 8 or not os.path.exists(path):
+        return None
+    entry = json.load(open(path)).get("workloads", {}).get(workload)
+    return entry["traffic_bytes"] if entry else None
+
+
 def timed_steps(wl, steps, warmup):
     """W untimed steps, then K timed ones between device synchronisations; every timed launch is also
     bracketed by GPU events on the launch stream."""
@@ -314,7 +324,8 @@ def main():
         peak, unit = PEAK[wl.dtype]
         achieved = wl.flops / (launch_ms * 1e-3) / 1e12
     roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "achieved": round(achieved, 2), "peak": peak,
-                "unit": unit, "frac": round(achieved / peak, 4), "traffic": None, "kernel": kernel,
+                "unit": unit, "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload, args.world),
+                "kernel": kernel,
                 "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(per_launch_ms), 5),
                 "algorithmic_bytes": bytes_alg, "algorithmic_flops": wl.flops}
 
