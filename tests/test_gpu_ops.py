@@ -95,6 +95,24 @@ def test_all_reduce_bit_exact(path, variant, mode, rank):
         assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
 
 
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+@pytest.mark.parametrize("W,rank", [(2, 1), (3, 0), (5, 4), (12, 7), (16, 15)])
+def test_all_reduce_other_world_sizes(path, W, rank):
+    """World sizes other than the register-cached peer counts (1, 3, 7 peers), including more than
+    eight slots, take the general peer loop."""
+    dtype = torch.bfloat16
+    M, N, K = 256, 128, 64
+    ctx = _ctx(W, rank, heap=1 << 24)
+    A, B = randint_cpu((M, K), 10, dtype), randint_cpu((K, N), 11, dtype)
+    peers = [randn_cpu((M, N), 100 + r, dtype) for r in range(W)]
+    for variant in ("one_shot", "two_shot"):
+        cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+        dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg, path=path)
+        exp = oracle.matmul_all_reduce(A, B, peers, rank, W, 64, 64, variant)
+        for r, got in enumerate(slot_copies(ctx, dC)):
+            assert_bits_equal(got, exp["C"][r], f"{kernel} {variant} W={W} slot {r}")
+
+
 def test_all_reduce_closed_form():
     """Rank r contributes r + 1 everywhere: every element sums to W(W+1)/2
     (the reference's tile-collective check, tests/context/test_all_reduce.py:245-246,352-356)."""
