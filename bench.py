@@ -26,7 +26,7 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s")}
+PEAK = {"hbm": (8000.0, "GB/s"), "bf16": (2500.0, "TFLOP/s"), "fp16": (2500.0, "TFLOP/s"), "fp8": (5000.0, "TFLOP/s")}
 
 
 def _randn(shape, seed, dtype, scale=1.0, device="cpu"):
@@ -49,10 +49,11 @@ class Workload:
 
 
 class MatmulAllReduce(Workload):
-    def __init__(self, name, M, N, K, fp8=False, block_m=256, variant="one_shot"):
+    def __init__(self, name, M, N, K, fp8=False, block_m=256, variant="one_shot", fp16=False):
         self.name, self.M, self.N, self.K, self.fp8 = name, M, N, K, fp8
         self.block_m, self.variant = block_m, variant
-        self.dtype = "fp8" if fp8 else "bf16"
+        self.dtype = "fp8" if fp8 else ("fp16" if fp16 else "bf16")
+        self.elem = torch.float16 if fp16 else torch.bfloat16  # type of C, aux and the peers' partials
         self.flops = 2 * M * N * K
 
     def algorithmic_bytes(self, world):
@@ -76,21 +77,21 @@ class MatmulAllReduce(Workload):
             self.scale = dict(scale_a=sa, scale_b=sb)
         else:
             g = torch.Generator().manual_seed(0)
-            A = (torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16)
-            B = (torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16)
+            A = (torch.randn((M, K), generator=g) / K ** 0.5).to(self.elem)
+            B = (torch.randn((K, N), generator=g) / K ** 0.5).to(self.elem)
         self.A_cpu, self.B_cpu = A, B
         self.A = ctx.zeros((M, K), dtype=A.dtype)
         self.A.copy_(A)
         self.B = ctx.zeros((K, N), dtype=B.dtype)
         self.B.copy_(B)
-        self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
+        self.C = ctx.zeros((M, N), dtype=self.elem)
         self.cfg = iris.FusedConfig(block_size_m=self.block_m, block_size_n=64, block_size_k=64,
                                     all_reduce_variant=self.variant)
         self.ws = ops.matmul_all_reduce_preamble(ctx, self.C, self.A, self.B, config=self.cfg)
         gen = torch.Generator(device="cuda").manual_seed(1)
         for r in range(1, world):  # synthetic peer partials, N(0,1) in bf16, flags raised
             ctx.peer_view(self.ws.aux_buffer, r).copy_(
-                torch.randn((M, N), generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16))
+                torch.randn((M, N), generator=gen, device="cuda", dtype=torch.float32).to(self.elem))
             ctx.peer_view(self.ws.locks, r).fill_(1)
         self._op = ops.matmul_all_reduce
         torch.cuda.synchronize()
@@ -256,6 +257,15 @@ WORKLOADS = {
     "matmul_all_reduce_fp8_skinny_32x8192x1024": lambda: MatmulAllReduce(
         "matmul_all_reduce_fp8_skinny_32x8192x1024", 32, 8192, 1024, fp8=True, block_m=32),
 }
+# Shapes of the reference's own benchmark definitions (no published results): fused vs unfused stages
+# at decode/prefill sizes (benchmark/ops/bench_matmul_all_reduce_stages.py:50-69: M in {32, 896, 2048},
+# N = 2880, K = 4096 / 8 ranks, fp16) and the large grid (benchmark/ops/bench_matmul_all_reduce.py:12-47).
+for _m in (32, 896, 2048):
+    WORKLOADS[f"matmul_all_reduce_fp16_{_m}x2880x512"] = (
+        lambda m=_m: MatmulAllReduce(f"matmul_all_reduce_fp16_{m}x2880x512", m, 2880, 512, fp16=True, block_m=32, variant="two_shot"))
+for _m in (1024, 4096, 16384):
+    WORKLOADS[f"matmul_all_reduce_fp16_{_m}x3584x8192"] = (
+        lambda m=_m: MatmulAllReduce(f"matmul_all_reduce_fp16_{m}x3584x8192", m, 3584, 8192, fp16=True, variant="two_shot"))
 DEFAULT = "matmul_all_reduce_bf16_4096x4096x1376"
 
 
