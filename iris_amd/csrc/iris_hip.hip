@@ -1121,16 +1121,30 @@ int dispatch_generic(const FusedParams& p, int in_dtype, int out_dtype, int cu, 
   return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
 }
 
-// Tile shapes of the MFMA kernel.  The large tile keeps 256 accumulator registers per lane busy;
-// the small one gives short problems enough workgroups to cover the 256 CUs.
+// Tile shapes of the MFMA kernel.
+//   big     256x256, 8 waves, 4-slot ring: 128 accumulator registers per lane, the shape for large
+//           problems (it alone fills the 256 CUs).
+//   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
+//   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
+// Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
+// smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
+enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2 };
+constexpr int tile_bk(int kind, int in) {  // K elements per step
+  return (kind == TILE_BIG ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
+}
 template <int IN, bool BKC>
-using BigTile = MfmaCfg<IN, 256, 256, (IN == IN_FP8 ? 64 : 32), 2, 4, 4, BKC>;
+using BigTile = MfmaCfg<IN, 256, 256, tile_bk(TILE_BIG, IN), 2, 4, 4, BKC>;
 template <int IN, bool BKC>
-using SmallTile = MfmaCfg<IN, 128, 128, (IN == IN_FP8 ? 64 : 32), 2, 2, 4, BKC>;
+using SmallTile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL, IN), 2, 2, 4, BKC>;
+template <int IN, bool BKC>
+using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
+
+inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SMALL ? 128 : 64; }
+inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : 128; }
 
 template <int IN>
-int dispatch_mfma_in(FusedParams& p, bool big, bool bkc, int cu, hipStream_t s) {
-  const int bm = big ? 256 : 128, bn = bm;
+int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int cu, hipStream_t s) {
+  const int bm = tile_rows(kind), bn = tile_cols(kind);
   p.tiles_m = cdiv(p.M, bm);
   p.tiles_n = cdiv(p.N, bn);
   // Group height: tile-rows walked together so that an XCD's span of tiles is close to square.
@@ -1140,13 +1154,15 @@ int dispatch_mfma_in(FusedParams& p, bool big, bool bkc, int cu, hipStream_t s) 
   p.group_m = g;
   static const char* names[3] = {"bf16", "f16", "fp8"};
   char name[96];
-  snprintf(name, sizeof(name), "mfma_%s_%dx%dx%d_%s", names[IN], bm, bn, IN == IN_FP8 ? 64 : 32, bkc ? "nt" : "nn");
-  if (big) {
-    if (bkc) return launch_mfma<BigTile<IN, true>>(p, cu, s, name);
-    return launch_mfma<BigTile<IN, false>>(p, cu, s, name);
+  snprintf(name, sizeof(name), "mfma_%s_%dx%dx%d_%s", names[IN], bm, bn, tile_bk(kind, IN), bkc ? "nt" : "nn");
+  switch (kind) {
+    case TILE_BIG:
+      return bkc ? launch_mfma<BigTile<IN, true>>(p, cu, s, name) : launch_mfma<BigTile<IN, false>>(p, cu, s, name);
+    case TILE_SMALL:
+      return bkc ? launch_mfma<SmallTile<IN, true>>(p, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, cu, s, name);
+    default:
+      return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, cu, s, name);
   }
-  if (bkc) return launch_mfma<SmallTile<IN, true>>(p, cu, s, name);
-  return launch_mfma<SmallTile<IN, false>>(p, cu, s, name);
 }
 
 int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
@@ -1174,19 +1190,21 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   p.num_xcd = facts->xcc_count;
   hipStream_t s = (hipStream_t)stream;
 
-  // Tile choice: the 256x256 tile when it alone fills most of the machine, else 128x128.
+  // Tile choice: the 256x256 tile when it alone fills most of the machine, 64-row tiles for
+  // decode-sized M, else 128x128.
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
-  const bool big = big_tiles * 10 >= (long long)facts->cu_count * 8;
-  const int bm = big ? 256 : 128;
-  const char* why = mfma_ineligible(p, in_dtype, out_dtype, bm, bm);
+  int kind = TILE_SMALL;
+  if (big_tiles * 10 >= (long long)facts->cu_count * 8) kind = TILE_BIG;
+  else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
+  const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
 
   const bool bkc = (p.s_bn != 1);
   switch (in_dtype) {
-    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, big, bkc, facts->cu_count, s);
-    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, big, bkc, facts->cu_count, s);
-    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, big, bkc, facts->cu_count, s);
+    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, kind, bkc, facts->cu_count, s);
+    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, kind, bkc, facts->cu_count, s);
+    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, kind, bkc, facts->cu_count, s);
   }
   return fail("unsupported input type %d", in_dtype);
 }
