@@ -279,12 +279,32 @@ def measured_traffic(workload, world):
     return entry["traffic_bytes"] if entry else None
 
 
-def timed_steps(wl, steps, warmup):
+def timed_steps(wl, steps, warmup, graph=False):
     """W untimed steps, then K timed ones between device synchronisations; every timed launch is also
-    bracketed by GPU events on the launch stream."""
+    bracketed by GPU events on the launch stream.  With graph=True the K steps are captured into one
+    HIP graph after the warm-up and the timed region is one replay of it (no host work between the
+    launches; the per-launch time is then the replay time divided by K)."""
     for _ in range(warmup):
         wl.step()
     torch.cuda.synchronize()
+    if graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        captured = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(captured, stream=side):
+            for _ in range(steps):
+                wl.step()
+        captured.replay()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        start.record()
+        captured.replay()
+        end.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        wl.ctx.check_status()
+        return wall, [start.elapsed_time(end) / steps] * steps
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     t0 = time.perf_counter()
@@ -308,6 +328,7 @@ def main():
     ap.add_argument("--world", type=int, default=8, help="number of heap slots W")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm-phase", action="store_true", help="skip the W=1 measurement")
+    ap.add_argument("--graph", action="store_true", help="capture the K steps into one HIP graph and time its replay")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build runs the rank-local path of one MI355X "
@@ -320,7 +341,7 @@ def main():
 
     wl = WORKLOADS[args.workload]()
     wl.setup(iris, args.world)
-    wall, per_launch_ms = timed_steps(wl, args.steps, args.warmup)
+    wall, per_launch_ms = timed_steps(wl, args.steps, args.warmup, args.graph)
     kernel = _lib.last_kernel() if not isinstance(wl, CopyCalibration) else "torch copy kernel"
     ms_per_step = wall * 1e3 / args.steps
     launch_ms = statistics.mean(per_launch_ms)
@@ -352,6 +373,7 @@ def main():
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
+        "launch_mode": "hip graph replay" if args.graph else "eager",
         "config": wl.describe(args.world),
         "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2) if wl.dtype in PEAK else None,
         "roofline": roofline,
@@ -362,7 +384,7 @@ def main():
         torch.cuda.empty_cache()
         solo = WORKLOADS[args.workload]()
         solo.setup(iris, 1)  # W = 1: same kernel and shape, no peers to sum
-        wall1, per1 = timed_steps(solo, args.steps, args.warmup)
+        wall1, per1 = timed_steps(solo, args.steps, args.warmup, args.graph)
         t1 = solo.flops * args.steps / wall1 / 1e12
         out["gemm_phase"] = {"world": 1, "tflops": round(t1, 3), "ms_per_step": round(wall1 * 1e3 / args.steps, 5),
                              "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4), "kernel": _lib.last_kernel()}

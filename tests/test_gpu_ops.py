@@ -414,3 +414,52 @@ def test_c_abi_rejects_bad_arguments():
     cu, xcc, lds = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int32()
     assert lib.iris_hip_query(0, ctypes.byref(cu), ctypes.byref(xcc), ctypes.byref(lds)) == 0
     assert cu.value == torch.cuda.get_device_properties(0).multi_processor_count and xcc.value >= 1
+
+
+# ------------------------------------------------------------------------------------------------
+# HIP graphs: a launch is one kernel node, so launch-bound loops can be captured and replayed
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+def test_graph_replay_matches_eager(variant):
+    W, dtype = 4, torch.bfloat16
+    M, N, K = 256, 384, 160
+    ctx = _ctx(W)
+    B = randint_cpu((K, N), 21, dtype)
+    peers = [randn_cpu((M, N), 200 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+    dA, dB = ctx.zeros((M, K), dtype=dtype), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    stage_peers(ctx, ws, peers)
+
+    def launch():
+        ws.prepared = True
+        ops.matmul_all_reduce(ctx, dC, dA, dB, async_op=True, config=cfg, workspace=ws)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()  # first call outside the capture: one-time function attributes are set here
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch()
+
+    for rep in range(4):
+        A = randint_cpu((M, K), 300 + rep, dtype)
+        dA.copy_(A)  # eager work between the replays: new operands, outputs and own flags cleared
+        for r in range(W):
+            ctx.peer_view(dC, r).zero_()
+        ws.locks.zero_()
+        ws.aux_buffer.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ctx.check_status()
+        exp = oracle.matmul_all_reduce(A, B, peers, 0, W, 64, 64, variant, "fp32")
+        assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"aux, replay {rep}")
+        assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), f"flags, replay {rep}"
+        got = slot_copies(ctx, dC)
+        for r in range(W):
+            assert_bits_equal(got[r], exp["C"][r], f"C in slot {r}, replay {rep}")
