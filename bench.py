@@ -245,6 +245,53 @@ class CopyCalibration(Workload):
         return None
 
 
+class CclCollective(Workload):
+    """Stand-alone all-reduce / reduce-scatter over the heap slots: one rank's launch, no GEMM.  The
+    value is reported in TFLOP/s like every other line (one fp32 add per input element), the roofline
+    in GB/s of the bytes the launch has to move."""
+
+    bound = "hbm"
+
+    def __init__(self, name, op, variant, M, N):
+        self.name, self.op, self.variant, self.M, self.N = name, op, variant, M, N
+
+    def _share(self, world):
+        return 1.0 if self.variant == "one_shot" else 1.0 / world  # fraction of the tiles the rank reduces
+
+    def algorithmic_bytes(self, world):
+        tile_bytes = self.M * self.N * 2 * self._share(world)
+        stores = world if (self.op == "all_reduce" and self.variant == "two_shot") else 1
+        return int(tile_bytes * (world + stores))
+
+    def describe(self, world):
+        return {"workload": self.name, "op": "ccl." + self.op, "variant": self.variant, "M": self.M, "N": self.N,
+                "W": world, "tile": [32, 64], "distribution": "block"}
+
+    def setup(self, iris, world):
+        from iris_amd.ccl import Config
+        M, N = self.M, self.N
+        self.flops = int(M * N * world * self._share(world))
+        self.ctx = ctx = iris.iris(4 * M * N + (16 << 20), num_ranks=world, rank=0)
+        self.x = ctx.zeros((M, N), dtype=torch.bfloat16)
+        self.y = ctx.zeros((M, N), dtype=torch.bfloat16)
+        gen = torch.Generator(device="cuda").manual_seed(3)
+        for r in range(world):
+            ctx.peer_view(self.x, r).copy_(torch.randn((M, N), generator=gen, device="cuda").to(torch.bfloat16))
+        self.cfg = Config(all_reduce_variant=self.variant)
+        self.ws = ctx.ccl.all_reduce_preamble(self.y, self.x, config=self.cfg) if self.op == "all_reduce" else None
+        torch.cuda.synchronize()
+
+    def step(self):
+        if self.op == "all_reduce":
+            self.ws.prepared = True  # the timed step is the launch; zeroing is the preamble's job
+            self.ctx.ccl.all_reduce(self.y, self.x, async_op=True, config=self.cfg, workspace=self.ws)
+        else:
+            self.ctx.ccl.reduce_scatter(self.y, self.x, async_op=True, config=self.cfg)
+
+    def cpu_baseline(self, world, budget_s=20.0):
+        return None
+
+
 WORKLOADS = {
     "copy_calibration_1GiB": lambda: CopyCalibration("copy_calibration_1GiB", 1 << 30),
     "matmul_all_reduce_bf16_4096x4096x1376": lambda: MatmulAllReduce("matmul_all_reduce_bf16_4096x4096x1376", 4096, 4096, 1376),
@@ -257,6 +304,13 @@ WORKLOADS = {
     "matmul_all_reduce_fp8_skinny_32x8192x1024": lambda: MatmulAllReduce(
         "matmul_all_reduce_fp8_skinny_32x8192x1024", 32, 8192, 1024, fp8=True, block_m=32),
 }
+for _v in ("one_shot", "two_shot"):
+    WORKLOADS[f"ccl_all_reduce_{_v}_bf16_8192x8192"] = (
+        lambda v=_v: CclCollective(f"ccl_all_reduce_{v}_bf16_8192x8192", "all_reduce", v, 8192, 8192))
+WORKLOADS["ccl_reduce_scatter_bf16_8192x8192"] = (
+    lambda: CclCollective("ccl_reduce_scatter_bf16_8192x8192", "reduce_scatter", "two_shot", 8192, 8192))
+WORKLOADS["ccl_all_reduce_one_shot_bf16_128x8192"] = (
+    lambda: CclCollective("ccl_all_reduce_one_shot_bf16_128x8192", "all_reduce", "one_shot", 128, 8192))
 # Shapes of the reference's own benchmark definitions (no published results): fused vs unfused stages
 # at decode/prefill sizes (benchmark/ops/bench_matmul_all_reduce_stages.py:50-69: M in {32, 896, 2048},
 # N = 2880, K = 4096 / 8 ranks, fp16) and the large grid (benchmark/ops/bench_matmul_all_reduce.py:12-47).

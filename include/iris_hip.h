@@ -169,6 +169,62 @@ int iris_hip_matmul_all_gather(const void* A, const void* B, void* C_gathered, c
                                int32_t in_dtype, int32_t out_dtype, int32_t bias_dtype, float scale,
                                int32_t path, void* stream);
 
+/* Tile-to-rank distribution of the two-shot collectives (Config.all_reduce_distribution,
+ * iris/ccl/config.py:42-43). */
+enum {
+  IRIS_HIP_DISTRIBUTION_STRIDED = 0, /* rank r owns tiles r, r+W, r+2W, ...                      */
+  IRIS_HIP_DISTRIBUTION_BLOCK = 1    /* rank r owns tiles [r*ceil(T/W), min((r+1)*ceil(T/W), T)) */
+};
+
+/*
+ * Stand-alone all-reduce over the symmetric heap: output = sum over the group's ranks of input,
+ * rank-local part.  Replaces the launches in iris/ccl/triton/all_reduce.py:762-956 of
+ *   persistent_all_reduce_atomic    (:120-215)  variant IRIS_HIP_VARIANT_ATOMIC
+ *   persistent_all_reduce_one_shot  (:345-423)  variant IRIS_HIP_VARIANT_ONE_SHOT
+ *   persistent_all_reduce_two_shot  (:574-706)  variant IRIS_HIP_VARIANT_TWO_SHOT
+ * with the arguments of those launches, in order, then variant, distribution, element type, stream.
+ *
+ * input and output are M x N tensors in the slot of `iris_rank` (strides in elements); the copy in
+ * the slot of rank q sits at the same heap offset.  The group is the ranks
+ * rank_start + i*rank_stride, i in [0, world_size); group_rank is this rank's index in it.
+ *   one_shot: every element = cast(fp32 sum of the group's inputs, in group order, starting from 0),
+ *             stored to the own output.
+ *   two_shot: tile ids run over the block_size_m x block_size_n grid in the grouped order of
+ *             swizzle_size tile-rows (all_reduce.py:628-633).  The rank reduces the tiles the
+ *             distribution gives it; the j-th of them (j = 0, 1, ...) is summed in fp32 starting at
+ *             group index (j mod comm_sms) mod world_size and going round cyclically (:663-669), cast
+ *             once, and stored to the output of every rank of the group.
+ *   atomic:   the own input is added atomically into the output of every rank of the group
+ *             (outputs must have been zeroed; all_reduce.py:83-85).
+ * comm_sms takes part in the two-shot summation order as above; the launch itself sizes its grid to
+ * the machine.  num_xcds and chunk_size are accepted for signature parity and change no result.
+ * dtype is IRIS_HIP_BF16, IRIS_HIP_FP16 or IRIS_HIP_FP32 (input and output alike).
+ */
+int iris_hip_all_reduce(const void* input, void* output, int64_t M, int64_t N,
+                        int64_t stride_in_m, int64_t stride_in_n,
+                        int64_t stride_out_m, int64_t stride_out_n,
+                        const int64_t* heap_bases,
+                        int32_t group_rank, int32_t iris_rank, int32_t world_size,
+                        int32_t rank_start, int32_t rank_stride,
+                        int32_t block_size_m, int32_t block_size_n, int32_t swizzle_size,
+                        int32_t comm_sms, int32_t num_xcds, int32_t chunk_size,
+                        int32_t variant, int32_t distribution, int32_t dtype, void* stream);
+
+/*
+ * Stand-alone reduce-scatter over the symmetric heap, rank-local part: the two-shot reduction above
+ * with the result stored to the own output only.  Replaces the launch of
+ * persistent_reduce_scatter_two_shot (iris/ccl/triton/reduce_scatter.py:160-190; kernel :16-140).
+ */
+int iris_hip_reduce_scatter(const void* input, void* output, int64_t M, int64_t N,
+                            int64_t stride_in_m, int64_t stride_in_n,
+                            int64_t stride_out_m, int64_t stride_out_n,
+                            const int64_t* heap_bases,
+                            int32_t group_rank, int32_t iris_rank, int32_t world_size,
+                            int32_t rank_start, int32_t rank_stride,
+                            int32_t block_size_m, int32_t block_size_n, int32_t swizzle_size,
+                            int32_t comm_sms, int32_t num_xcds, int32_t chunk_size,
+                            int32_t distribution, int32_t dtype, void* stream);
+
 /*
  * Device facts used by the host layer (reference: get_cu_count / get_num_xcc,
  * iris/host/platform/hip.py:138,218).  Any output pointer may be NULL.

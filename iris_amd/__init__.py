@@ -9,7 +9,7 @@ The package keeps the reference's Python surface (context, tensor factories, hea
 signatures) and runs hand-written gfx950 kernels from libiris_hip.so underneath.
 """
 
-from . import ops
+from . import ccl, ops
 from .host.bench import do_bench
 from .host.iris import Iris, iris
 from .host.logging import DEBUG, ERROR, INFO, WARNING, logger, set_logger_level
@@ -19,6 +19,7 @@ __all__ = [
     "iris",
     "Iris",
     "ops",
+    "ccl",
     "FusedConfig",
     "FusedWorkspace",
     "do_bench",

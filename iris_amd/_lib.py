@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # IRIS_HIP_LIBRARY names another build of the same library (e.g. one compiled with other tile shapes).
 LIBRARY_PATH = os.environ.get("IRIS_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libiris_hip.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # Enumerations of include/iris_hip.h
 BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
@@ -20,6 +20,7 @@ ACC_FP32, ACC_REFERENCE = 0, 1
 GATHER_K, GATHER_M = 1, 2
 PATH_AUTO, PATH_MFMA, PATH_GENERIC = 0, 1, 2
 STATUS_SPIN_TIMEOUT = 1
+DISTRIBUTION_STRIDED, DISTRIBUTION_BLOCK = 0, 1
 
 _i32, _i64, _f32, _ptr = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -28,6 +29,11 @@ _GEMM_HEAD = [_ptr, _ptr, _ptr, _ptr, _ptr,  # A, B, C, aux_buffer, locks
               _i64, _i64, _i64, _i64, _i64, _i64,  # strides am ak bk bn cm cn
               _ptr, _i32, _i32,  # context_tensor, cur_rank, world_size
               _i32, _i32, _i32]  # block sizes m n k
+
+_CCL_HEAD = [_ptr, _ptr, _i64, _i64,  # input, output, M, N
+             _i64, _i64, _i64, _i64,  # strides in_m in_n out_m out_n
+             _ptr, _i32, _i32, _i32, _i32, _i32,  # heap_bases, group_rank, iris_rank, world_size, rank_start, rank_stride
+             _i32, _i32, _i32, _i32, _i32, _i32]  # block m, block n, swizzle_size, comm_sms, num_xcds, chunk_size
 
 PROTOTYPES = {
     "iris_hip_matmul_all_reduce": (
@@ -63,6 +69,8 @@ PROTOTYPES = {
          _i32, _i32, _i32, _f32,  # in_dtype, out_dtype, bias_dtype, scale
          _i32, _ptr],  # path, stream
     ),
+    "iris_hip_all_reduce": (_i32, _CCL_HEAD + [_i32, _i32, _i32, _ptr]),  # variant, distribution, dtype, stream
+    "iris_hip_reduce_scatter": (_i32, _CCL_HEAD + [_i32, _i32, _ptr]),  # distribution, dtype, stream
     "iris_hip_query": (_i32, [_i32, _ptr, _ptr, _ptr]),
     "iris_hip_last_error": (ctypes.c_char_p, []),
     "iris_hip_last_kernel": (ctypes.c_char_p, []),
@@ -100,3 +108,12 @@ def last_error():
 
 def last_kernel():
     return library().iris_hip_last_kernel().decode("utf-8")
+
+
+def query(device):
+    """(cu_count, xcc_count, lds_bytes_per_block) of GPU `device`."""
+    cu, xcc, lds = _i32(), _i32(), _i32()
+    err = library().iris_hip_query(device, ctypes.byref(cu), ctypes.byref(xcc), ctypes.byref(lds))
+    if err:
+        raise RuntimeError(f"HIP error code {err}: {last_error()}")
+    return cu.value, xcc.value, lds.value

@@ -12,8 +12,9 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-SOURCES = [os.path.join(HERE, "iris_hip.hip")]
-HEADERS = [os.path.join(HERE, "layout.h"), os.path.join(ROOT, "include", "iris_hip.h")]
+SOURCES = [os.path.join(HERE, "iris_hip.hip"), os.path.join(HERE, "iris_ccl.hip")]
+HEADERS = [os.path.join(HERE, h) for h in ("layout.h", "device_util.h", "host_common.h")] + [
+    os.path.join(ROOT, "include", "iris_hip.h")]
 OUTPUT = os.path.join(os.path.dirname(HERE), "lib", "libiris_hip.so")
 
 FLAGS = [

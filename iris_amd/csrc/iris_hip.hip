@@ -30,6 +30,8 @@
 
 #include "iris_hip.h"
 #include "layout.h"
+#include "device_util.h"
+#include "host_common.h"
 
 using namespace iris_layout;
 
@@ -76,62 +78,12 @@ struct FusedParams {
   int* status;
   int tiles_m, tiles_n, group_m, num_xcd;
   int row_offset;  // all-gather: first row of this rank's block in the gathered output
+  int stream_peers;  // phase 2 reads the peers' tiles and writes C with non-temporal accesses
 };
 
 // ------------------------------------------------------------------------------------------------
 // Small device helpers
 // ------------------------------------------------------------------------------------------------
-
-// Address of `p` (a pointer into slot `from`) in slot `to`.
-__device__ __forceinline__ char* slot_ptr(const long long* heap_bases, const void* p, int from, int to) {
-  unsigned long long off = (unsigned long long)p - (unsigned long long)heap_bases[from];
-  return (char*)((unsigned long long)heap_bases[to] + off);
-}
-
-__device__ __forceinline__ float bf16_bits_to_float(unsigned short b) { return __uint_as_float(((unsigned)b) << 16); }
-
-__device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
-  __bf16 h = (__bf16)f;  // round to nearest even; v_cvt_pk_bf16_f32 on gfx950
-  return __builtin_bit_cast(unsigned short, h);
-}
-__device__ __forceinline__ unsigned short float_to_f16_bits(float f) {
-  _Float16 h = (_Float16)f;
-  return __builtin_bit_cast(unsigned short, h);
-}
-__device__ __forceinline__ float f16_bits_to_float(unsigned short b) {
-  return (float)__builtin_bit_cast(_Float16, b);
-}
-
-// Output element kinds of the 16-bit epilogue.
-struct OutBF16 {
-  static __device__ __forceinline__ float to_float(unsigned short b) { return bf16_bits_to_float(b); }
-  static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_bf16_bits(f); }
-  static constexpr bool kFp32SumInReference = false;
-};
-struct OutF16 {
-  static __device__ __forceinline__ float to_float(unsigned short b) { return f16_bits_to_float(b); }
-  static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_f16_bits(f); }
-  static constexpr bool kFp32SumInReference = true;
-};
-
-// Atomically add two packed 16-bit floats (one 32-bit word) to memory.
-typedef __attribute__((ext_vector_type(2))) short s16x2_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
-template <class Out>
-__device__ __forceinline__ void atomic_add_packed(char* addr, unsigned word) {
-  if constexpr (Out::kFp32SumInReference)  // float16
-    __builtin_amdgcn_global_atomic_fadd_v2f16((__attribute__((address_space(1))) f16x2_t*)addr,
-                                              __builtin_bit_cast(f16x2_t, word));
-  else
-    __builtin_amdgcn_global_atomic_fadd_v2bf16((__attribute__((address_space(1))) s16x2_t*)addr,
-                                               __builtin_bit_cast(s16x2_t, word));
-}
-
-__device__ __forceinline__ float load_scalar_as_float(const char* base, long long idx, int dtype) {
-  if (dtype == IRIS_HIP_FP32) return ((const float*)base)[idx];
-  unsigned short b = ((const unsigned short*)base)[idx];
-  return dtype == IRIS_HIP_BF16 ? bf16_bits_to_float(b) : f16_bits_to_float(b);
-}
 
 __device__ __forceinline__ int owner_of(int epi, int t, int total, int world, int rank) {
   if (epi == EPI_TWO_SHOT) return owner_interleaved(t, world);
@@ -723,8 +675,9 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       for (int i = 0; i < kMaxCachedSlots - 1; ++i) pb[i] = (i < p.rank ? hb[i] : hb[i + 1]) + (aux_own - hb_own);
       const long long safe_off = ((long long)m0 * p.s_cm + n0) * 2;  // first element of the tile
 
-      auto reduce_tile = [&](auto np_tag) {
+      auto reduce_tile = [&](auto np_tag, auto nt_tag) {
         constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
+        constexpr bool NT = decltype(nt_tag)::value;  // peers' tiles and C bypass the caches' keep policy
         constexpr int NPV = NP > 0 ? NP : 1;
         constexpr int G = NP >= 4 ? 2 : 4;           // passes whose loads are issued together
         static_assert(PASSES % G == 0, "pass grouping");
@@ -745,7 +698,10 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
             eoff[g] = active[g] ? ((long long)gm * p.s_cm + gn) * 2 : safe_off;
             if constexpr (NP > 0) {
 #pragma unroll
-              for (int i = 0; i < NP; ++i) pv[g][i] = *(const u32x4_t*)(pb[i] + eoff[g]);
+              for (int i = 0; i < NP; ++i) {
+                if constexpr (NT) pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
+                else pv[g][i] = *(const u32x4_t*)(pb[i] + eoff[g]);
+              }
             }
             own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
           }
@@ -786,7 +742,9 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
                   if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
               } else {
                 const int dst = p.all_owners ? owner[g] : p.rank;
-                *(u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]) = res;
+                u32x4_t* cdst = (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]);
+                if constexpr (NT) __builtin_nontemporal_store(res, cdst);
+                else *cdst = res;
               }
             }
           }
@@ -794,10 +752,16 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
       };
       switch (solo ? -2 : (p.world <= kMaxCachedSlots ? npeers : -1)) {
         case -2: break;  // C was written in phase 1
-        case 1: reduce_tile(std::integral_constant<int, 1>{}); break;
-        case 3: reduce_tile(std::integral_constant<int, 3>{}); break;
-        case 7: reduce_tile(std::integral_constant<int, 7>{}); break;
-        default: reduce_tile(std::integral_constant<int, -1>{}); break;
+        case 1: reduce_tile(std::integral_constant<int, 1>{}, std::false_type{}); break;
+        case 3: reduce_tile(std::integral_constant<int, 3>{}, std::false_type{}); break;
+        case 7:
+          // Peer tiles are read once; when they exceed what the last-level cache holds, streaming
+          // them non-temporally is faster (measured: 663 -> 622 us for 7 x 256 MiB of peers), for
+          // smaller launches it is not (two-shot 4096 x 4096: 91 -> 98 us).
+          if (p.stream_peers) reduce_tile(std::integral_constant<int, 7>{}, std::true_type{});
+          else reduce_tile(std::integral_constant<int, 7>{}, std::false_type{});
+          break;
+        default: reduce_tile(std::integral_constant<int, -1>{}, std::false_type{}); break;
       }
     }
     // Staging shares LDS with the operand ring of the next tile.
@@ -808,54 +772,6 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
 // ------------------------------------------------------------------------------------------------
 // Generic kernel: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMA.
 // ------------------------------------------------------------------------------------------------
-// Atomic add of one 16-bit float: compare-and-swap on the aligned 32-bit word that contains it.
-template <class E>
-__device__ __forceinline__ void atomic_add_half(char* p, float f) {
-  unsigned* word = (unsigned*)((unsigned long long)p & ~3ull);
-  const int shift = ((unsigned long long)p & 2) ? 16 : 0;
-  unsigned old = *word, assumed;
-  do {
-    assumed = old;
-    unsigned short cur = (unsigned short)(assumed >> shift);
-    float sum = E::load((const char*)&cur) + f;
-    unsigned short nv;
-    E::store((char*)&nv, sum);
-    const unsigned repl = (assumed & ~(0xFFFFu << shift)) | ((unsigned)nv << shift);
-    old = atomicCAS(word, assumed, repl);
-  } while (old != assumed);
-}
-
-struct ElemBF16 {
-  static constexpr int size = 2;
-  static __device__ __forceinline__ float load(const char* p) { return bf16_bits_to_float(*(const unsigned short*)p); }
-  static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_bf16_bits(f); }
-  static __device__ __forceinline__ float round(float f) { return bf16_bits_to_float(float_to_bf16_bits(f)); }
-  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomic_add_half<ElemBF16>(p, f); }
-  static constexpr bool kFp32SumInReference = false;
-};
-struct ElemF16 {
-  static constexpr int size = 2;
-  static __device__ __forceinline__ float load(const char* p) { return f16_bits_to_float(*(const unsigned short*)p); }
-  static __device__ __forceinline__ void store(char* p, float f) { *(unsigned short*)p = float_to_f16_bits(f); }
-  static __device__ __forceinline__ float round(float f) { return f16_bits_to_float(float_to_f16_bits(f)); }
-  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomic_add_half<ElemF16>(p, f); }
-  static constexpr bool kFp32SumInReference = true;
-};
-struct ElemF32 {
-  static constexpr int size = 4;
-  static __device__ __forceinline__ float load(const char* p) { return *(const float*)p; }
-  static __device__ __forceinline__ void store(char* p, float f) { *(float*)p = f; }
-  static __device__ __forceinline__ float round(float f) { return f; }
-  static __device__ __forceinline__ void atomic_add(char* p, float f) { atomicAdd((float*)p, f); }
-  static constexpr bool kFp32SumInReference = false;  // fp32 data sums in fp32 either way
-};
-struct ElemFP8 {
-  static constexpr int size = 1;
-  static __device__ __forceinline__ float load(const char* p) {
-    return __builtin_amdgcn_cvt_f32_fp8((int)*(const unsigned char*)p, 0);
-  }
-};
-
 constexpr int GT = 64;   // generic tile edge
 constexpr int GK = 16;   // generic k step
 
@@ -1200,6 +1116,8 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
 
+  p.stream_peers = epi_has_flags(p.epi) && p.sum_peers &&
+                   (long long)(p.world - 1) * p.M * p.N * 2 > (512ll << 20);
   const bool bkc = (p.s_bn != 1);
   switch (in_dtype) {
     case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, kind, bkc, facts->cu_count, s);
@@ -1212,6 +1130,31 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
 bool fits_int(int64_t v) { return v > 0 && v < (1ll << 31); }
 
 }  // namespace
+
+namespace iris_host {
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return (int)hipErrorInvalidValue;
+}
+
+void clear_last_error() { g_last_error[0] = 0; }
+
+void set_last_kernel(const char* name) { snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name); }
+
+int device_facts(int device, int* cu_count, int* xcc_count) {
+  DeviceFacts* f = nullptr;
+  const int rc = facts_for(device, &f);
+  if (rc) return rc;
+  *cu_count = f->cu_count;
+  *xcc_count = f->xcc_count;
+  return 0;
+}
+
+}  // namespace iris_host
 
 extern "C" {
 
@@ -1344,6 +1287,6 @@ int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }
-int iris_hip_abi_version(void) { return 2; }
+int iris_hip_abi_version(void) { return 3; }
 
 }  // extern "C"

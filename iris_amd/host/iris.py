@@ -80,6 +80,7 @@ class Iris:
         self.device = str(self.heap.device) if backing == "host" else f"cuda:{self.gpu_id}"
         self.heap_bases = self.heap.get_heap_bases()
         self._ops = None
+        self._ccl = None
         self._cu_count = None
         # Flag-wait bound handed to the kernels (polls per flag; <= 0 waits forever as the reference).
         self.spin_limit = int(os.environ.get("IRIS_SPIN_LIMIT", str(1 << 22)))
@@ -119,6 +120,43 @@ class Iris:
 
             self._ops = OpsNamespace(self)
         return self._ops
+
+    @property
+    def ccl(self):
+        """Stand-alone collectives bound to this context (`ctx.ccl.all_reduce(output, input)`)."""
+        if self._ccl is None:
+            self._ccl = Iris.CCL(self)
+        return self._ccl
+
+    class CCL:
+        """The `ctx.ccl` namespace of the reference (iris/host/iris.py:1104-1311), for the collectives
+        that have HIP kernels here: all_reduce (+ preamble) and reduce_scatter."""
+
+        def __init__(self, iris_instance):
+            self._iris = iris_instance
+
+        def all_reduce_preamble(self, output_tensor, input_tensor, config=None, workspace=None):
+            from ..ccl.all_reduce import all_reduce_preamble
+
+            return all_reduce_preamble(output_tensor, input_tensor, self._iris, config=config, workspace=workspace)
+
+        def all_reduce(self, output_tensor, input_tensor, op=None, group=None, async_op=False, config=None,
+                       workspace=None):
+            from ..ccl.all_reduce import all_reduce
+
+            return all_reduce(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
+                              config=config, workspace=workspace)
+
+        def reduce_scatter(self, output_tensor, input_tensor, op=None, group=None, async_op=False, config=None):
+            from ..ccl.reduce_scatter import reduce_scatter
+
+            reduce_scatter(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
+                           config=config)
+
+        def __getattr__(self, name):
+            if name in ("all_to_all", "all_gather"):
+                raise NotImplementedError(f"ccl.{name} has no HIP kernel in this package")
+            raise AttributeError(name)
 
     # -- tensor factories --------------------------------------------------------------------------
     def _dev(self):

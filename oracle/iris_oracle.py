@@ -30,6 +30,15 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
                                                  tests/ops/test_all_gather_matmul.py:61-66)
   flag contents                                 source-pinned only (no reference test asserts them):
                                                  parity unpinned by tests
+  ccl_owned_tiles, ccl_tile_coords              pinned: partition property (every tile owned exactly once
+                                                 over the ranks, both distributions), bijection of the
+                                                 grouped order, and hand-worked small grids
+  ccl_all_reduce / ccl_reduce_scatter           pinned: closed form "rank r holds r+1 => W(W+1)/2"
+                                                 (tests/ccl/test_all_reduce.py:55,92-97), equality with a
+                                                 plain fp32 sum for exactly representable data, and the
+                                                 one-shot order against a sequential Python sum.  The
+                                                 rotated start rank of two-shot is source-pinned only (no
+                                                 reference test can see it): parity unpinned by tests
   quantize_e4m3 / fp8 products                  no reference counterpart (the reference has no fp8
                                                  path): defined by BASELINE's config 5, parity unpinned
 """
@@ -289,6 +298,106 @@ def matmul_all_gather(A, B, rank, world, bias=None, out_dtype=None, scale=1.0):
 # ----------------------------------------------------------------------------------------------
 # Error measure used by the parity tests
 # ----------------------------------------------------------------------------------------------
+
+
+# ----------------------------------------------------------------------------------------------
+# Stand-alone collectives (iris.ccl)
+# ----------------------------------------------------------------------------------------------
+
+
+def ccl_tile_coords(tile, tiles_m, tiles_n, group_m):
+    """(pid_m, pid_n) of tile id `tile` in the grouped order.
+
+    iris/ccl/triton/all_reduce.py:639-644:
+        num_pid_in_group = GROUP_SIZE_M * num_pid_n; group_id = tile_id // num_pid_in_group
+        first_pid_m = group_id * GROUP_SIZE_M; group_size_m = min(num_pid_m - first_pid_m, GROUP_SIZE_M)
+        pid_m = first_pid_m + ((tile_id % num_pid_in_group) % group_size_m)
+        pid_n = (tile_id % num_pid_in_group) // group_size_m
+    """
+    per_group = group_m * tiles_n
+    group = tile // per_group
+    first = group * group_m
+    size = min(tiles_m - first, group_m)
+    return first + (tile % per_group) % size, (tile % per_group) // size
+
+
+def ccl_owned_tiles(total_tiles, group_rank, world, distribution):
+    """Tile ids rank `group_rank` reduces, in the order j = 0, 1, ... the kernel's loop meets them.
+
+    iris/ccl/triton/all_reduce.py:620-633 (the same lines in iris/ccl/triton/reduce_scatter.py:58-70):
+    distribution 0 strides (rank, rank+W, ...), distribution 1 takes ceil(T/W) consecutive tiles.
+    """
+    per_rank = cdiv(total_tiles, world)
+    if distribution == 0:
+        return list(range(group_rank, total_tiles, world))
+    start = group_rank * per_rank
+    return list(range(start, min(start + per_rank, total_tiles)))
+
+
+def _ccl_cast_sum(slices, order, from_zero):
+    acc = torch.zeros_like(slices[0], dtype=torch.float32) if from_zero else None
+    for r in order:
+        x = slices[r].to(torch.float32)
+        acc = x.clone() if acc is None else acc + x
+    return acc
+
+
+def ccl_all_reduce(inputs, outputs, group_rank, variant, block_m=32, block_n=64, group_m=4, comm_sms=64,
+                   distribution=1):
+    """What the launch of rank `group_rank` leaves in every rank's output.
+
+    inputs / outputs: lists (one entry per rank of the group, group order) of (M, N) tensors; outputs
+    are the contents before the launch and are not modified.  Returns the new list of outputs.
+
+    one_shot (iris/ccl/triton/all_reduce.py:401-422): acc = zeros fp32; acc += input of rank i for
+        i = 0..W-1; own output = cast(acc).
+    two_shot (:646-684): for the j-th owned tile, start = pid % W where the loop gives
+        j = pid (mod COMM_SMS); acc = fp32(input[start]); acc += input[(start+i) % W], i = 1..W-1;
+        cast once; stored to the output of every rank.
+    atomic (:210-233): the own input is added into every rank's output (in the output's type).
+    """
+    world = len(inputs)
+    M, N = inputs[0].shape
+    dtype = inputs[0].dtype
+    outs = [o.clone() for o in outputs]
+    if variant == "atomic":
+        for r in range(world):
+            outs[r] = (outs[r].to(torch.float32) + inputs[group_rank].to(torch.float32)).to(dtype)
+        return outs
+    if variant == "one_shot":
+        outs[group_rank] = _ccl_cast_sum(inputs, range(world), True).to(dtype)
+        return outs
+    if variant != "two_shot":
+        raise ValueError(variant)
+    reduced = ccl_reduce_scatter(inputs, outputs[group_rank], group_rank, block_m, block_n, group_m, comm_sms,
+                                 distribution, _mask_out=True)
+    tile, mask = reduced
+    for r in range(world):
+        outs[r] = torch.where(mask, tile, outs[r])
+    return outs
+
+
+def ccl_reduce_scatter(inputs, output, group_rank, block_m=32, block_n=64, group_m=4, comm_sms=64, distribution=1,
+                       _mask_out=False):
+    """The own output after the launch of rank `group_rank`: owned tiles hold the cast fp32 sum, the
+    rest keeps `output` (iris/ccl/triton/reduce_scatter.py:72-118; same reduction as two-shot
+    all-reduce, stored to the own rank only)."""
+    world = len(inputs)
+    M, N = inputs[0].shape
+    dtype = inputs[0].dtype
+    tiles_m, tiles_n = cdiv(M, block_m), cdiv(N, block_n)
+    out = output.clone()
+    mask = torch.zeros((M, N), dtype=torch.bool)
+    for j, tile in enumerate(ccl_owned_tiles(tiles_m * tiles_n, group_rank, world, distribution)):
+        pid_m, pid_n = ccl_tile_coords(tile, tiles_m, tiles_n, group_m)
+        rows = slice(pid_m * block_m, min((pid_m + 1) * block_m, M))
+        cols = slice(pid_n * block_n, min((pid_n + 1) * block_n, N))
+        start = (j % comm_sms) % world
+        order = [(start + i) % world for i in range(world)]
+        acc = _ccl_cast_sum([x[rows, cols] for x in inputs], order, False)
+        out[rows, cols] = acc.to(dtype)
+        mask[rows, cols] = True
+    return (out, mask) if _mask_out else out
 
 
 def rel_frobenius(x, ref):

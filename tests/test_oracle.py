@@ -244,3 +244,94 @@ def test_all_reduce_atomic_variant():
         C = oracle.matmul_all_reduce(As[rank], B, C, rank, W, 4, 4, "atomic")["C"]
     for r in range(W):
         assert torch.equal(C[r], sum(a @ B for a in As))
+
+
+# ------------------------------------------------------------------------------------------------
+# Stand-alone collectives
+# ------------------------------------------------------------------------------------------------
+def test_ccl_grouped_order_hand_worked():
+    # 3 x 2 tiles, groups of 2 tile-rows: the first group is walked column by column (two rows per
+    # column), the last group has a single row.
+    got = [oracle.ccl_tile_coords(t, 3, 2, 2) for t in range(6)]
+    assert got == [(0, 0), (1, 0), (0, 1), (1, 1), (2, 0), (2, 1)]
+    # one tile-row per group is plain row-major order
+    assert [oracle.ccl_tile_coords(t, 2, 3, 1) for t in range(6)] == [(0, 0), (0, 1), (0, 2), (1, 0), (1, 1), (1, 2)]
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n,group_m", [(1, 1, 4), (5, 3, 4), (8, 8, 4), (7, 2, 3), (4, 9, 6)])
+def test_ccl_grouped_order_is_a_bijection(tiles_m, tiles_n, group_m):
+    seen = {oracle.ccl_tile_coords(t, tiles_m, tiles_n, group_m) for t in range(tiles_m * tiles_n)}
+    assert seen == {(m, n) for m in range(tiles_m) for n in range(tiles_n)}
+
+
+@pytest.mark.parametrize("distribution", [0, 1])
+@pytest.mark.parametrize("total,world", [(1, 4), (7, 4), (8, 8), (33, 8), (64, 3), (5, 16)])
+def test_ccl_ownership_partitions_the_tiles(total, world, distribution):
+    owned = [oracle.ccl_owned_tiles(total, r, world, distribution) for r in range(world)]
+    flat = sorted(t for tiles in owned for t in tiles)
+    assert flat == list(range(total)), "every tile reduced by exactly one rank"
+    if distribution == 0:
+        assert all(t % world == r for r, tiles in enumerate(owned) for t in tiles)
+    else:
+        per = -(-total // world)
+        assert all(t // per == r for r, tiles in enumerate(owned) for t in tiles)
+
+
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot", "atomic"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_ccl_all_reduce_closed_form(variant, dtype):
+    # tests/ccl/test_all_reduce.py:55: rank r holds r+1 everywhere, so every element is W(W+1)/2
+    W, M, N = 8, 128, 128
+    inputs = [torch.full((M, N), float(r + 1), dtype=dtype) for r in range(W)]
+    outs = [torch.zeros((M, N), dtype=dtype) for _ in range(W)]
+    for r in range(W):  # every rank runs its launch
+        outs = oracle.ccl_all_reduce(inputs, outs, r, variant, block_m=32, block_n=32, distribution=r % 2 if variant != "two_shot" else 0)
+    for r in range(W):
+        assert torch.all(outs[r] == W * (W + 1) / 2)
+
+
+@pytest.mark.parametrize("distribution", [0, 1])
+def test_ccl_two_shot_over_all_ranks_is_the_plain_sum(distribution):
+    W, M, N = 4, 100, 72  # ragged against 32 x 64 tiles
+    g = torch.Generator().manual_seed(5)
+    inputs = [torch.randint(-8, 9, (M, N), generator=g).to(torch.bfloat16) for _ in range(W)]
+    outs = [torch.full((M, N), -1.0, dtype=torch.bfloat16) for _ in range(W)]
+    for r in range(W):
+        outs = oracle.ccl_all_reduce(inputs, outs, r, "two_shot", distribution=distribution)
+    want = sum(x.float() for x in inputs).to(torch.bfloat16)  # small integers: exact in any order
+    for r in range(W):
+        assert torch.equal(outs[r], want)
+    # reduce-scatter: each rank's owned tiles agree with the sum, the rest is untouched
+    covered = torch.zeros((M, N), dtype=torch.int32)
+    for r in range(W):
+        own = oracle.ccl_reduce_scatter(inputs, torch.full((M, N), -1.0, dtype=torch.bfloat16), r, distribution=distribution)
+        touched = own != -1.0
+        assert torch.equal(own[touched], want[touched])
+        covered += touched.int()
+    assert torch.all(covered[want != -1.0] == 1)
+
+
+def test_ccl_one_shot_adds_in_group_order_from_zero():
+    # fp32 values whose sum depends on the order: 2^24 + 1 + 1 - 2^24
+    vals = [2.0 ** 24, 1.0, 1.0, -(2.0 ** 24)]
+    inputs = [torch.full((4, 8), v, dtype=torch.float32) for v in vals]
+    outs = [torch.zeros((4, 8)) for _ in vals]
+    got = oracle.ccl_all_reduce(inputs, outs, 2, "one_shot")[2]
+    acc = np.float32(0.0)
+    for v in vals:
+        acc = np.float32(acc + np.float32(v))
+    assert acc == 0.0 and torch.all(got == float(acc))  # the two ones are absorbed one at a time
+    # -0.0 in every slot comes out as +0.0 because the accumulator starts from +0.0
+    neg = [torch.full((2, 8), -0.0, dtype=torch.bfloat16) for _ in range(4)]
+    out = oracle.ccl_all_reduce(neg, [torch.ones((2, 8), dtype=torch.bfloat16)] * 4, 0, "one_shot")[0]
+    assert torch.all(out.view(torch.int16) == 0)
+
+
+def test_ccl_two_shot_with_one_workgroup_starts_every_tile_at_rank_zero():
+    # comm_sms = 1 makes (j mod comm_sms) mod W zero for every tile: the order is the ascending one
+    vals = [2.0 ** 24, 1.0, 1.0, -(2.0 ** 24)]
+    inputs = [torch.full((64, 64), v, dtype=torch.float32) for v in vals]
+    outs = [torch.zeros((64, 64)) for _ in vals]
+    for r in range(4):
+        outs = oracle.ccl_all_reduce(inputs, outs, r, "two_shot", block_m=32, block_n=32, comm_sms=1, distribution=0)
+    assert all(torch.all(o == 0.0) for o in outs)
