@@ -85,6 +85,9 @@ class Iris:
         # Flag-wait bound handed to the kernels (polls per flag; <= 0 waits forever as the reference).
         self.spin_limit = int(os.environ.get("IRIS_SPIN_LIMIT", str(1 << 22)))
         self._status = torch.zeros(1, dtype=torch.int32, device=self.heap.device)
+        # One GPU standing in for all ranks: when set, the fused operators' preambles mark the other
+        # ranks as finished (flags raised, aux zeroed) so that a launch does not wait for them.
+        self.stand_in_peers = os.environ.get("IRIS_STAND_IN_PEERS", "0") not in ("", "0")
         self._build_device_context()
 
     def __del__(self):

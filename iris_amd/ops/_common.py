@@ -78,3 +78,22 @@ def iris_launch(entry_name, grid, *args, algorithm, rank, dtype=None):
         log_rank(logging.ERROR, "HIP error code %d: %s", err, text, rank=rank)
         raise RuntimeError(f"HIP error code {err}: {text}")
     return None
+
+
+def stage_idle_peers(shmem, workspace):
+    """One GPU standing in for all ranks: make the other ranks look finished with nothing to add.
+
+    Called by the preambles when the context has `stand_in_peers` set (the benchmark harness sets it):
+    the peers' flags are raised and their aux buffers zeroed, so that a fused launch neither waits for
+    ranks that do not run nor sums uninitialised memory.  The reference has no counterpart - its peers
+    are live processes.
+    """
+    if not getattr(shmem, "stand_in_peers", False):
+        return
+    for r in range(shmem.get_num_ranks()):
+        if r == shmem.get_rank():
+            continue
+        if workspace.locks is not None:
+            shmem.peer_view(workspace.locks, r).fill_(1)
+        if workspace.aux_buffer is not None:
+            shmem.peer_view(workspace.aux_buffer, r).zero_()

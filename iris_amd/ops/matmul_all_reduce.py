@@ -13,7 +13,7 @@ import torch
 from .. import _lib
 from ..host.logging import log_rank
 from ._common import (acc_code, current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr,
-                      require_gpu_tensors)
+                      require_gpu_tensors, stage_idle_peers)
 from .config import FusedConfig
 from .workspace import FusedWorkspace
 
@@ -70,6 +70,7 @@ def matmul_all_reduce_preamble(
         workspace.aux_buffer = None
 
     C.zero_()
+    stage_idle_peers(shmem, workspace)
     shmem.barrier()
     workspace.prepared = True
     return workspace

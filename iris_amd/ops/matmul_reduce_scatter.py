@@ -12,7 +12,7 @@ import torch
 
 from ..host.logging import log_rank
 from ._common import (acc_code, current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr,
-                      require_gpu_tensors)
+                      require_gpu_tensors, stage_idle_peers)
 from .config import FusedConfig
 from .workspace import FusedWorkspace
 
@@ -67,6 +67,7 @@ def matmul_reduce_scatter_preamble(
     else:
         workspace.aux_buffer.zero_()
     C.zero_()
+    stage_idle_peers(shmem, workspace)
     shmem.barrier()
     workspace.prepared = True
     return workspace
