@@ -92,9 +92,15 @@ __device__ __forceinline__ int owner_of(int epi, int t, int total, int world, in
 }
 
 // Raise the flags of the flag tiles covered by the macro tile at (m0, n0) of KM x KN elements.
-// Must be called by every thread of the workgroup after a release fence and a workgroup barrier
-// that follow the workgroup's aux stores.
-template <int KM, int KN, int NT>
+// Must be called by every thread of the workgroup after the workgroup's aux stores have completed
+// (vmcnt(0)) and a workgroup barrier.
+// WRITTEN_THROUGH = false: the aux stores were ordinary stores (dirty lines in L2), so the flag is
+//   raised with system-scope release, which writes the L2 back first.
+// WRITTEN_THROUGH = true: the aux stores were system-scope write-through stores (store16_system) that
+//   have been acknowledged, so the data is already where a peer reads it and a relaxed system-scope
+//   flag store after them is enough; this spares one whole-L2 write-back per workgroup (measured 5-11 %
+//   of the fused launch).
+template <int KM, int KN, int NT, bool WRITTEN_THROUGH>
 __device__ __forceinline__ void raise_flags(const FusedParams& p, int m0, int n0, int tid) {
   const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
   const int ftn = cdiv(p.N, p.flag_bn);
@@ -109,10 +115,14 @@ __device__ __forceinline__ void raise_flags(const FusedParams& p, int m0, int n0
     bool last = true;
     if (needed > 1) {
       // Arrivals are counted in steps of 2 so that the flag never reads 1 before the last one.
-      int old = __hip_atomic_fetch_add(flag, 2, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
+      int old = WRITTEN_THROUGH ? __hip_atomic_fetch_add(flag, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
+                                : __hip_atomic_fetch_add(flag, 2, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
       last = ((old >> 1) + 1) == needed;
     }
-    if (last) __hip_atomic_exchange(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (last) {
+      if (WRITTEN_THROUGH) __hip_atomic_exchange(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      else __hip_atomic_exchange(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
@@ -218,6 +228,12 @@ __device__ __forceinline__ void dma16(i32x4_t rsrc, unsigned lds_base, unsigned 
                :
                : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
+}
+
+// 16-byte store that is written through to memory at system scope (sc0 sc1): once vmcnt reports it
+// done, every agent that reads the address with a coherent load sees it, without an L2 write-back.
+__device__ __forceinline__ void store16_system(char* p, u32x4_t v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
 }
 
 // Read one accumulator register.  The "a" constraint keeps the MFMA results in the accumulation
@@ -626,6 +642,8 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
 #pragma unroll
               for (int e = 0; e < 4; ++e) atomic_add_packed<Out>(dst + 4 * e, v[e]);
             }
+          } else if (flags) {
+            store16_system(out1 + eoff, v);  // aux: read by the peers as soon as the flag is up
           } else {
             *(u32x4_t*)(out1 + eoff) = v;
           }
@@ -646,14 +664,14 @@ __global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p
     }
 
     if (flags) {
-      // Publish: every wave waits until its aux stores have reached L2, the workgroup meets, and
-      // the threads that raise flags do so with system-scope release (one L2 write-back per
-      // workgroup instead of one per wave).  Likewise the peers' flags are polled (system-scope
+      // Publish: the aux tile was stored write-through at system scope; every wave waits until its
+      // stores are acknowledged, the workgroup meets, and the threads that own flags raise them
+      // (no L2 write-back is needed any more).  Likewise the peers' flags are polled (system-scope
       // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
       // every wave poll and run ahead measured slower.
       wait_vmcnt<0>();
       __syncthreads();
-      raise_flags<BM, BN, NT>(p, m0, n0, tid);
+      raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
       if (!solo) {
         wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
         __syncthreads();
@@ -875,7 +893,7 @@ __global__ void __launch_bounds__(256) fused_generic_kernel(const FusedParams p)
 
     __atomic_thread_fence(__ATOMIC_RELEASE);
     __syncthreads();
-    raise_flags<GT, GT, 256>(p, m0, n0, tid);
+    raise_flags<GT, GT, 256, false>(p, m0, n0, tid);
     if (p.sum_peers && p.world > 1) {
       wait_peer_flags<GT, GT, 256>(p, m0, n0, tid);
       __syncthreads();
