@@ -6,17 +6,20 @@
 //  * fused_mfma_kernel  - persistent tiled GEMM on the 32x32 MFMA blocks of CDNA4.  Operand tiles
 //    travel HBM -> LDS with 16-byte direct-to-LDS buffer loads into a ring of STAGES buffers
 //    (prefetch distance STAGES-1, one workgroup barrier per K step); the K-contiguous operand is
-//    read back with 16-byte LDS reads, the N-contiguous one with LDS transpose reads.  Each of the
-//    four waves owns a (BM/2)x(BN/2) block of fp32 accumulators.  Requires 16-byte aligned,
-//    unit-stride rows (see mfma_eligible()).
+//    read back with 16-byte LDS reads, the N-contiguous one with LDS transpose reads.  The waves of
+//    a workgroup (8 as 2x4 for the 256x256 tile, 4 as 2x2 for the smaller ones) each own a block of
+//    fp32 accumulators that stays in the accumulation registers.  Requires 16-byte aligned,
+//    unit-stride rows (see mfma_ineligible()).
 //  * fused_generic_kernel - a plain 64x64 LDS-tiled FMA kernel for everything else (fp32 data,
 //    odd strides, sizes that are not multiples of 8 elements).
 //
-// Both end in the same epilogue protocol, which follows the reference kernels
+// The flag-less operators (all_gather_matmul, matmul_all_gather, the atomic all-reduce) store or add
+// the tile directly.  The others end in the same epilogue protocol, which follows the reference kernels
 // (iris/ops/matmul_all_reduce.py:111-144, iris/ops/matmul_reduce_scatter.py:98-118,
 //  iris/mem/triton/context.py:733-764, 801-839, 953-997):
 //    1. cast the fp32 tile to the output type and store it to aux in the own slot,
-//    2. make those stores visible, then raise the flag of every finished flag tile,
+//    2. make those stores visible, then raise the flag of every finished flag tile (the MFMA
+//       kernel writes aux through to memory and raises relaxed; the generic kernel raises with release),
 //    3. for the flag tiles this rank reduces: wait for the peers' flags, add the peers' aux tiles
 //       in ascending rank order, cast once, store to C (own slot; two-shot: every slot).
 
