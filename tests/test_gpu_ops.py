@@ -463,3 +463,40 @@ def test_graph_replay_matches_eager(variant):
         got = slot_copies(ctx, dC)
         for r in range(W):
             assert_bits_equal(got[r], exp["C"][r], f"C in slot {r}, replay {rep}")
+
+
+# ------------------------------------------------------------------------------------------------
+# Ragged extents on the MFMA path: partial tiles in M, N and K, single-row problems
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(200, 264, 72), (1000, 520, 1376), (1, 2880, 512), (33, 136, 24), (4100, 4104, 40)])
+@pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
+def test_ragged_shapes_mfma(M, N, K, variant):
+    W, rank, dtype = 8, 6, torch.bfloat16
+    ctx = _ctx(W, rank, heap=1 << 27)
+    A, B = randint_cpu((M, K), 50, dtype), randint_cpu((K, N), 51, dtype)
+    peers = [randn_cpu((M, N), 600 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=32 if M >= 32 else 1, block_size_n=64, block_size_k=8, all_reduce_variant=variant)
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg, path="mfma")
+    assert kernel.startswith("mfma_bf16"), kernel
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, cfg.block_size_m, cfg.block_size_n, variant, "fp32")
+    assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], "aux")
+    assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+    got = slot_copies(ctx, dC)
+    for r in range(W):
+        assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
+
+
+@pytest.mark.parametrize("M,N,K", [(200, 272, 80), (1, 1024, 256), (520, 144, 1008)])
+def test_ragged_shapes_mfma_fp8(M, N, K):
+    W, rank = 4, 1
+    ctx = _ctx(W, rank)
+    a, b = randn_cpu((M, K), 60, torch.float32), randn_cpu((K, N), 61, torch.float32)
+    (Aq, sa), (Bq, sb) = oracle.quantize_e4m3(a), oracle.quantize_e4m3(b)
+    peers = [randn_cpu((M, N), 700 + r, torch.bfloat16) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=32 if M >= 32 else 1, block_size_n=64, block_size_k=16, all_reduce_variant="one_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, Aq, Bq, peers, cfg, path="mfma", out_dtype=torch.bfloat16, scale_a=sa, scale_b=sb)
+    assert kernel.startswith("mfma_fp8"), kernel
+    exp = oracle.matmul_all_reduce(Aq, Bq, peers, rank, W, cfg.block_size_m, 64, "one_shot", "fp32",
+                                   out_dtype=torch.bfloat16, scale=sa * sb)
+    assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+    assert oracle.rel_frobenius(dC.cpu(), exp["C"][rank]) < 3e-2
