@@ -190,6 +190,10 @@ struct MfmaCfg {
   static constexpr int TILE_BYTES = BM * TROW;
   static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES;
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+  // Four-wave tiles whose ring fits twice into a CU's LDS run two workgroups per CU, so that the
+  // memory round trips of one workgroup's epilogue hide behind the other's K loop.
+  static constexpr int WG_PER_CU = (NW == 4 && SMEM_BYTES <= 80 * 1024) ? 2 : 1;
+  static constexpr int WAVES_PER_SIMD = WG_PER_CU * NW / 4;
   static_assert(NT % (BN / 8) == 0 && BM % (NT / (BN / 8)) == 0, "epilogue pass shape");
   static_assert(A_BYTES % (kDmaBytes * NW) == 0 && B_BYTES % (kDmaBytes * NW) == 0, "tile/loader mismatch");
   static_assert(BK % KM == 0 && TM % 32 == 0 && TN % 32 == 0, "tile/MFMA mismatch");
@@ -289,7 +293,7 @@ constexpr int kMaxCachedSlots = 8;  // heap bases kept in registers; larger worl
 // MFMA kernel
 // ------------------------------------------------------------------------------------------------
 template <class CFG>
-__global__ void __launch_bounds__(CFG::NT) fused_mfma_kernel(const FusedParams p) {
+__global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kernel(const FusedParams p) {
   using Out = typename OutOf<CFG::IN>::type;
   using ATile = RowTile<CFG::RBA>;
   constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
@@ -1025,7 +1029,8 @@ int launch_mfma(const FusedParams& p, int cu_count, hipStream_t stream, const ch
     attr_set = true;
   }
   const int total = p.tiles_m * p.tiles_n;
-  int grid = total < cu_count ? total : cu_count;
+  const int cap = cu_count * CFG::WG_PER_CU;
+  int grid = total < cap ? total : cap;
   if (grid >= p.num_xcd) grid -= grid % p.num_xcd;  // keep the XCD mapping exact
   if (grid < 1) grid = 1;
   hipLaunchKernelGGL(fused_mfma_kernel<CFG>, dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
@@ -1060,14 +1065,18 @@ int dispatch_generic(const FusedParams& p, int in_dtype, int out_dtype, int cu, 
 
 // Tile shapes of the MFMA kernel.
 //   big     256x256, 8 waves, 4-slot ring: 128 accumulator registers per lane, the shape for large
-//           problems (it alone fills the 256 CUs).
+//           problems (half the operand bytes per flop of the 128x128 tiles).
 //   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
 //   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
 // Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
 // smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
-enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2 };
+//   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
+//           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
+//           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
+//           tiles the shorter K steps make it the slower of the two.
+enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
-  return (kind == TILE_BIG ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
+  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
 }
 template <int IN, bool BKC>
 using BigTile = MfmaCfg<IN, 256, 256, tile_bk(TILE_BIG, IN), 2, 4, 4, BKC>;
@@ -1075,8 +1084,10 @@ template <int IN, bool BKC>
 using SmallTile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL, IN), 2, 2, 4, BKC>;
 template <int IN, bool BKC>
 using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
+template <int IN, bool BKC>
+using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
 
-inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SMALL ? 128 : 64; }
+inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SKINNY ? 64 : 128; }
 inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : 128; }
 
 template <int IN>
@@ -1097,6 +1108,8 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int cu, hipStream_t s) 
       return bkc ? launch_mfma<BigTile<IN, true>>(p, cu, s, name) : launch_mfma<BigTile<IN, false>>(p, cu, s, name);
     case TILE_SMALL:
       return bkc ? launch_mfma<SmallTile<IN, true>>(p, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, cu, s, name);
+    case TILE_SMALL2:
+      return bkc ? launch_mfma<Small2Tile<IN, true>>(p, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, cu, s, name);
     default:
       return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, cu, s, name);
   }
@@ -1127,12 +1140,14 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   p.num_xcd = facts->xcc_count;
   hipStream_t s = (hipStream_t)stream;
 
-  // Tile choice: the 256x256 tile when it alone fills most of the machine, 64-row tiles for
-  // decode-sized M, else 128x128.
+  // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
+  // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64-row tiles for decode-sized M, else
+  // 128x128 - two workgroups per CU when there are more such tiles than CUs.
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
-  if (big_tiles * 10 >= (long long)facts->cu_count * 8) kind = TILE_BIG;
+  if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
   else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
+  else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
   const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
