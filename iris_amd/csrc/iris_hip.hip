@@ -10,7 +10,7 @@
 //    a workgroup (8 as 2x4 for the 256x256 tile, 4 as 2x2 for the smaller ones) each own a block of
 //    fp32 accumulators that stays in the accumulation registers.  Requires 16-byte aligned,
 //    unit-stride rows (see mfma_ineligible()).
-//  * fused_generic_kernel - a plain 64x64 LDS-tiled FMA kernel for everything else (fp32 data,
+//  * fused_generic_kernel - a plain 64x64 LDS-tiled kernel on fp32 MFMA for everything else (fp32 data,
 //    odd strides, sizes that are not multiples of 8 elements).
 //
 // The flag-less operators (all_gather_matmul, matmul_all_gather, the atomic all-reduce) store or add
@@ -804,8 +804,15 @@ template <class In, class Out>
 __global__ void __launch_bounds__(256) fused_generic_kernel(const FusedParams p) {
   __shared__ float As[GK][GT + 1];
   __shared__ float Bs[GK][GT + 1];
+  __shared__ float Cs[GT][GT + 1];
   const int tid = threadIdx.x;
   const int tx = tid % 16, ty = tid / 16;
+  // Each of the four waves multiplies one 32x32 quadrant of the tile with fp32 MFMA
+  // (v_mfma_f32_32x32x2_f32: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32] of a 32x2 by 2x32
+  // product); inputs of every type are widened to fp32 in LDS first, so products are exact for 16-bit
+  // and fp8 data and accumulation is fp32 throughout.
+  const int lane = tid & 63, wave = tid >> 6;
+  const int qm = (wave >> 1) * 32, qn = (wave & 1) * 32;
   const int total_tiles = p.tiles_m * p.tiles_n;
   const int ftn = cdiv(p.N, p.flag_bn);
   const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
@@ -815,59 +822,72 @@ __global__ void __launch_bounds__(256) fused_generic_kernel(const FusedParams p)
   for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
     const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
     const int m0 = tm * GT, n0 = tn * GT;
+    f32x16_t quad;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) quad[r] = 0.f;
+
+    // One K step = GK columns of A and rows of B.  The operands of step t+1 are fetched into
+    // registers while the MFMAs of step t run, and stored to LDS after them.
+    const int ksteps = cdiv(klocal, GK);
+    const int nsteps = nsrc * ksteps;
+    auto fetch = [&](int step, float (&va)[4], float (&vb)[4]) {
+      const int src = step / ksteps, k0 = (step - src * ksteps) * GK;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {  // A tile: GT rows x GK k
+        const int idx = tid + e * 256;
+        const int r = idx / GK, kk = idx % GK;
+        const int gm = m0 + r, kl = k0 + kk;
+        va[e] = 0.f;
+        if (gm < p.M && kl < klocal) {
+          int slot = p.rank;
+          long long row = gm;
+          if (p.gather == GATHER_K) slot = src;
+          if (p.gather == GATHER_M) { slot = gm / p.M_local; row = gm - (long long)slot * p.M_local; }
+          const char* base = p.gather == GATHER_NONE ? p.A : slot_ptr(p.heap_bases, p.A, p.rank, slot);
+          va[e] = In::load(base + (row * p.s_am + (long long)kl * p.s_ak) * In::size);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {  // B tile: GK k x GT columns
+        const int idx = tid + e * 256;
+        const int kk = idx / GT, c = idx % GT;
+        const int gn = n0 + c, kl = k0 + kk;
+        vb[e] = 0.f;
+        if (gn < p.N && kl < klocal) {
+          const long long kg = (long long)src * klocal + kl;
+          vb[e] = In::load(p.B + (kg * p.s_bk + (long long)gn * p.s_bn) * In::size);
+        }
+      }
+    };
+    float va[4], vb[4];
+    fetch(0, va, vb);
+    for (int step = 0; step < nsteps; ++step) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int idx = tid + e * 256;
+        As[idx % GK][idx / GK] = va[e];
+        Bs[idx / GT][idx % GT] = vb[e];
+      }
+      __syncthreads();
+      if (step + 1 < nsteps) fetch(step + 1, va, vb);
+#pragma unroll
+      for (int kk = 0; kk < GK; kk += 2) {
+        const float a = As[kk + (lane >> 5)][qm + (lane & 31)];
+        const float b = Bs[kk + (lane >> 5)][qn + (lane & 31)];
+        quad = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, quad, 0, 0, 0);
+      }
+      __syncthreads();
+    }
+    // Accumulator register r of lane l is element (8*(r/4) + 4*(l/32) + r%4, l%32) of the quadrant;
+    // the tile goes through LDS so that the epilogue below can work on 4x4 blocks per thread.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) Cs[qm + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4)][qn + (lane & 31)] = quad[r];
+    __syncthreads();
     float acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
-
-    for (int src = 0; src < nsrc; ++src) {
-      for (int k0 = 0; k0 < klocal; k0 += GK) {
-        // A tile: GT rows x GK k; thread loads 4 elements.
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int idx = tid + e * 256;  // 0..1023
-          const int r = idx / GK, kk = idx % GK;
-          const int gm = m0 + r, kl = k0 + kk;
-          float v = 0.f;
-          if (gm < p.M && kl < klocal) {
-            int slot = p.rank;
-            long long row = gm;
-            if (p.gather == GATHER_K) slot = src;
-            if (p.gather == GATHER_M) { slot = gm / p.M_local; row = gm - (long long)slot * p.M_local; }
-            const char* base = p.gather == GATHER_NONE ? p.A : slot_ptr(p.heap_bases, p.A, p.rank, slot);
-            v = In::load(base + (row * p.s_am + (long long)kl * p.s_ak) * In::size);
-          }
-          As[kk][r] = v;
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int idx = tid + e * 256;
-          const int kk = idx / GT, c = idx % GT;
-          const int gn = n0 + c, kl = k0 + kk;
-          float v = 0.f;
-          if (gn < p.N && kl < klocal) {
-            const long long kg = (long long)src * klocal + kl;
-            v = In::load(p.B + (kg * p.s_bk + (long long)gn * p.s_bn) * In::size);
-          }
-          Bs[kk][c] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < GK; ++kk) {
-          float a[4], b[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
-        }
-        __syncthreads();
-      }
-    }
+      for (int j = 0; j < 4; ++j) acc[i][j] = Cs[ty * 4 + i][tx * 4 + j];
 
     // Own tile, rounded to the output type.
     float own[4][4];
