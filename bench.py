@@ -11,7 +11,7 @@ the fused kernel (HBM for the slot-sum workloads, MFMA for the others); `gemm_ph
 measurement with the peers switched off (W = 1), which isolates the MFMA phase; `cpu_baseline` times
 torch's CPU matmul plus the slot reduction on a bounded sample of the same workload.
 
-Default workload: BASELINE configuration 2, matmul_all_reduce bf16 M=N=4096, K=1376, W=8.
+Default workload: the headline configuration, matmul_all_reduce bf16 M=N=4096, K=1376, W=8.
 """
 
 import argparse

@@ -40,7 +40,8 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
                                                  rotated start rank of two-shot is source-pinned only (no
                                                  reference test can see it): parity unpinned by tests
   quantize_e4m3 / fp8 products                  no reference counterpart (the reference has no fp8
-                                                 path): defined by BASELINE's config 5, parity unpinned
+                                                 path): defined by the target configuration itself (e4m3fn inputs with
+                                                 per-tensor scales amax/448, fp32 accumulation), parity unpinned
 """
 
 import math

@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at full size on the GPU, against the CPU oracle.
+"""The five target configurations of this build at full size on the GPU, against the CPU oracle.
 
 Inputs are drawn on the CPU from torch.Generator().manual_seed(seed) as the configurations state.
 Full-size comparisons use the oracle directly where it finishes in seconds; the largest case (fp8,
