@@ -49,18 +49,26 @@ struct RowTile {
 };
 
 // ---------------------------------------------------------------------------------------------
-// Col tile: [BK rows][RB bytes], RB = BN*ES >= 256 (16-bit) or >= 128 (8-bit).  A 16-lane group
-// of a transpose read touches 4 k-rows x 32 B (16-bit) or 8 k-rows x 16 B (8-bit); rotating the
-// chunk index by the k-row keeps those on distinct banks.
+// Col tile: [BK rows][RB bytes], RB = BN*ES >= 256 (16-bit) or >= 128 (8-bit).  LDS serves a
+// transpose read one half-wave (32 lanes x 8 bytes = 256 bytes = all 64 banks) at a time.  A half-wave
+// touches 4 k-rows x 64 contiguous bytes (16-bit) or 8 k-rows x 32 bytes (8-bit); the other half-wave
+// reads the same columns 8 (32) k-rows further down.  XOR-ing the index of that 64- (32-) byte block
+// with the k-row puts the rows of a half-wave on distinct blocks of a 256-byte bank line.  When a
+// 256-byte bank line holds two tile rows (RB = 128) the row parity already separates them and the
+// XOR uses k-row / 2.  (Rotating 32-byte blocks by k-row % 8 for 16-bit data, as an earlier layout
+// did, is conflict-free per 16 lanes but lets rows 2i and 2i+1 of a half-wave share a block: the
+// hardware counted bank conflicts on half of the cycles of these reads.)
 // ---------------------------------------------------------------------------------------------
 template <int RB, int ES>
 struct ColTile {
   static_assert(ES == 1 || ES == 2, "element size must be 1 or 2 bytes");
   static constexpr int kChunksPerRow = RB / kChunkBytes;
-  static constexpr int kSw = (ES == 2) ? 2 : 1;
-  static_assert(kChunksPerRow >= 8 * kSw, "tile row too short for the swizzle");
+  static constexpr int kBlockChunks = (ES == 2) ? 4 : 2;        // 16-byte chunks per swizzled block
+  static constexpr int kRowsPerLine = RB >= 256 ? 1 : 256 / RB;  // tile rows per 256-byte bank line
+  static constexpr int kSwRows = ((ES == 2) ? 4 : 8) / kRowsPerLine;
+  static_assert(kChunksPerRow >= kSwRows * kBlockChunks, "tile row too short for the swizzle");
 
-  IRIS_HD static int swizzle(int krow) { return (krow % 8) * kSw; }
+  IRIS_HD static int swizzle(int krow) { return ((krow / kRowsPerLine) % kSwRows) * kBlockChunks; }
   IRIS_HD static int lds_offset(int krow, int c) { return krow * RB + ((c ^ swizzle(krow)) * kChunkBytes); }
   IRIS_HD static void from_lds(int off, int& krow, int& c) {
     krow = off / RB;

@@ -128,15 +128,15 @@ void sim_col_operand(int BK) {
       for (int rd = 0; rd < nreads; ++rd) {
         // every lane presents an address; the hardware redistributes within 16-lane groups
         int addr[64];
-        std::set<int> banks_by_group[4];
+        std::set<int> banks_by_group[2];  // LDS serves a transpose read one half-wave (256 bytes) at a time
         for (int lane = 0; lane < 64; ++lane) {
           int krow = ES == 2 ? tr16_krow(lane, kk, rd) : tr8_krow(lane, kk, rd);
           int n = n0 + (ES == 2 ? tr16_ncol(lane) : tr8_ncol(lane));
           addr[lane] = T::lds_offset(krow, n / CE) + (n % CE) * ES;
-          for (int b = 0; b < 8; b += 4) banks_by_group[lane / 16].insert(((addr[lane] + b) % 256) / 4);
+          for (int b = 0; b < 8; b += 4) banks_by_group[lane / 32].insert(((addr[lane] + b) % 256) / 4);
         }
-        for (int g = 0; g < 4; ++g)
-          CHECK(banks_by_group[g].size() == 32, "col operand ES=%d: bank conflict in lane group %d (%zu banks)", ES, g, banks_by_group[g].size());
+        for (int g = 0; g < 2; ++g)
+          CHECK(banks_by_group[g].size() == 64, "col operand ES=%d RB=%d: bank conflict in half-wave %d (%zu banks)", ES, RB, g, banks_by_group[g].size());
         for (int lane = 0; lane < 64; ++lane) {
           int grp = lane / 16, i = lane % 16;
           for (int e = 0; e < per_read; ++e) {
