@@ -34,6 +34,19 @@ def _randn(shape, seed, dtype, scale=1.0, device="cpu"):
     return (torch.randn(shape, generator=g, dtype=torch.float32) * scale).to(dtype)
 
 
+def _time_cpu(fn, flops, budget_s, sample):
+    """Median wall time of fn over 3..10 repetitions within budget_s seconds, as a cpu_baseline record."""
+    fn()
+    times, t_end = [], time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{sample}; {len(times)} reps, median; os.cpu_count={os.cpu_count()}"}
+
+
 class Workload:
     """One configuration: builds the heap tensors, launches a step, knows its flop and byte counts."""
 
@@ -166,7 +179,12 @@ class AllGatherMatmul(Workload):
         self._op(self.ctx, self.C, self.A, self.B, async_op=True, gather_dim=0)
 
     def cpu_baseline(self, world, budget_s=20.0):
-        return None
+        """torch CPU matmul of the first gathered row block (slot 0's rows) with B, bf16 in and out."""
+        rows = min(self.M // world, 1024)
+        A = _randn((rows, self.K), 0, torch.bfloat16, self.K ** -0.5)
+        B = _randn((self.K, self.N), 8, torch.bfloat16, self.K ** -0.5)
+        return _time_cpu(lambda: torch.matmul(A, B), 2 * rows * self.N * self.K, budget_s,
+                         f"first {rows} of {self.M} rows; torch.matmul bf16")
 
 
 class MatmulReduceScatter(Workload):
@@ -213,7 +231,14 @@ class MatmulReduceScatter(Workload):
         self._launch()
 
     def cpu_baseline(self, world, budget_s=20.0):
-        return None
+        """torch CPU matmul of the first 1024-row block plus its copy into the owner's output."""
+        rows = min(self.M, 1024)
+        g = torch.Generator().manual_seed(0)
+        A = (torch.randn((rows, self.K), generator=g) / self.K ** 0.5).to(torch.bfloat16)
+        B = (torch.randn((self.K, self.N), generator=g) / self.K ** 0.5).to(torch.bfloat16)
+        out = torch.empty((rows, self.N), dtype=torch.bfloat16)
+        return _time_cpu(lambda: out.copy_(torch.matmul(A, B)), 2 * rows * self.N * self.K, budget_s,
+                         f"first {rows} of {self.M} rows; torch.matmul bf16 + row-block copy")
 
 
 class CopyCalibration(Workload):
