@@ -1050,13 +1050,14 @@ const char* mfma_ineligible(const FusedParams& p, int in_dtype, int out_dtype, i
 }
 
 template <class CFG>
-int launch_mfma(const FusedParams& p, int cu_count, hipStream_t stream, const char* name) {
-  static bool attr_set = false;
-  if (!attr_set) {
+int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stream, const char* name) {
+  // The dynamic-LDS limit is a per-device attribute of the kernel: set it once on every device used.
+  static bool attr_set[64] = {};
+  if (!attr_set[device]) {
     hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
     if (e != hipSuccess) return (int)e;
-    attr_set = true;
+    attr_set[device] = true;
   }
   const int total = p.tiles_m * p.tiles_n;
   const int cap = cu_count * CFG::WG_PER_CU;
@@ -1121,7 +1122,7 @@ inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SK
 inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : 128; }
 
 template <int IN>
-int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int cu, hipStream_t s) {
+int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hipStream_t s) {
   const int bm = tile_rows(kind), bn = tile_cols(kind);
   p.tiles_m = cdiv(p.M, bm);
   p.tiles_n = cdiv(p.N, bn);
@@ -1135,13 +1136,13 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int cu, hipStream_t s) 
   snprintf(name, sizeof(name), "mfma_%s_%dx%dx%d_%s", names[IN], bm, bn, tile_bk(kind, IN), bkc ? "nt" : "nn");
   switch (kind) {
     case TILE_BIG:
-      return bkc ? launch_mfma<BigTile<IN, true>>(p, cu, s, name) : launch_mfma<BigTile<IN, false>>(p, cu, s, name);
+      return bkc ? launch_mfma<BigTile<IN, true>>(p, device, cu, s, name) : launch_mfma<BigTile<IN, false>>(p, device, cu, s, name);
     case TILE_SMALL:
-      return bkc ? launch_mfma<SmallTile<IN, true>>(p, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, cu, s, name);
+      return bkc ? launch_mfma<SmallTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, device, cu, s, name);
     case TILE_SMALL2:
-      return bkc ? launch_mfma<Small2Tile<IN, true>>(p, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, cu, s, name);
+      return bkc ? launch_mfma<Small2Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, device, cu, s, name);
     default:
-      return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, cu, s, name);
+      return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, device, cu, s, name);
   }
 }
 
@@ -1186,9 +1187,9 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
                    (long long)(p.world - 1) * p.M * p.N * 2 > (512ll << 20);
   const bool bkc = (p.s_bn != 1);
   switch (in_dtype) {
-    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, kind, bkc, facts->cu_count, s);
-    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, kind, bkc, facts->cu_count, s);
-    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, kind, bkc, facts->cu_count, s);
+    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, kind, bkc, device, facts->cu_count, s);
+    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, kind, bkc, device, facts->cu_count, s);
+    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, kind, bkc, device, facts->cu_count, s);
   }
   return fail("unsupported input type %d", in_dtype);
 }
