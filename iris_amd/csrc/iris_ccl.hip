@@ -340,6 +340,7 @@ int run_ccl(CclParams p, int distribution, int dtype, void* stream) {
     p.n_owned = (int)total;
   }
   p.upr = cdiv(p.bn, vec);
+  if ((long long)p.upr * p.bm >= (1ll << 31)) return fail("block sizes %d x %d are too large", p.bm, p.bn);
   p.upt = p.upr * p.bm;
   p.total_units = (long long)p.n_owned * p.upt;
 
