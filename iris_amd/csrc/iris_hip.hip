@@ -212,6 +212,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
+// The same with lgkmcnt(0): every LDS read of this wave has returned as well.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_lgkm0() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4));
+}
+
 constexpr unsigned kInvalidOffset = 0x80000000u;
 
 // Buffer resource words for a raw buffer (stride 0) over [base, base + 2^31).  Bounds are enforced
@@ -298,6 +304,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   using ATile = RowTile<CFG::RBA>;
   constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
   constexpr int MB = CFG::MB, NB = CFG::NB, TM = CFG::TM, TN = CFG::TN, NW = CFG::NW, NT = CFG::NT;
+  constexpr bool PINGPONG = CFG::NW == 8;
   constexpr int STAGES = CFG::STAGES, LA = CFG::LA, LB = CFG::LB, NFRAG = CFG::NFRAG, KS = CFG::KSLICES;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -393,8 +400,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   }
 
   // Read the fragments of k-slice kk of ring slot `slot`.
-  auto load_frags = [&](Frags<CFG>& f, int slot, int kk) {
-    const char* sa = smem + slot * CFG::STAGE_BYTES;
+  auto load_frags = [&](Frags<CFG>& f, int slot_off, int kk) {  // slot_off: byte offset of the ring slot
+    const char* sa = smem + slot_off;
     const char* sb = sa + CFG::A_BYTES;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -477,12 +484,12 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       int klim;
       unsigned sa, sb, a_soff, b_soff;
     };
-    auto begin_step = [&](int slot) {
+    auto begin_step = [&](int slot_off) {  // slot_off: byte offset of the ring slot to fill
       StepLoads L;
       const bool live = i_step < nsteps;
       const int k0 = i_kb * BK;
       L.klim = live ? klocal - k0 : 0;  // k elements of this step that exist
-      L.sa = smem_base + slot * CFG::STAGE_BYTES + wave * kDmaBytes;
+      L.sa = smem_base + slot_off + wave * kDmaBytes;
       L.sb = L.sa + CFG::A_BYTES;
       L.a_soff = (unsigned)(k0 * ES);
       const long long kglob = (long long)i_src * klocal + k0;
@@ -490,17 +497,19 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
       return L;
     };
-    auto issue_one = [&](const StepLoads& L, int j) {  // j in [0, LA + LB)
-      if (j < LA) {
-        const unsigned v = (la_k[j] < L.klim) ? a_voff[j] : kInvalidOffset;
-        dma16(ra, L.sa + j * NW * kDmaBytes, v, L.a_soff);
-      } else {
-        const int i = j - LA;
-        const int kpos = CFG::B_KCONTIG ? lb_col[i] : lb_row[i];
-        const unsigned v = (kpos < L.klim) ? b_voff[i] : kInvalidOffset;
-        dma16(rb, L.sb + i * NW * kDmaBytes, v, L.b_soff);
-      }
+    auto load_offset = [&](const StepLoads& L, int j) -> unsigned {  // per-lane offset of load j
+      if (j < LA) return (la_k[j] < L.klim) ? a_voff[j] : kInvalidOffset;
+      const int i = j - LA;
+      const int kpos = CFG::B_KCONTIG ? lb_col[i] : lb_row[i];
+      return (kpos < L.klim) ? b_voff[i] : kInvalidOffset;
     };
+    auto issue_at = [&](const StepLoads& L, int j, unsigned v) {
+      if (j < LA)
+        dma16(ra, L.sa + j * NW * kDmaBytes, v, L.a_soff);
+      else
+        dma16(rb, L.sb + (j - LA) * NW * kDmaBytes, v, L.b_soff);
+    };
+    auto issue_one = [&](const StepLoads& L, int j) { issue_at(L, j, load_offset(L, j)); };  // j in [0, LA + LB)
     auto end_step = [&]() {
       ++i_step;
       if (++i_kb == nkb) {  // next source slot (gather along K only)
@@ -510,7 +519,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       }
     };
     auto issue = [&](int slot) {
-      const StepLoads L = begin_step(slot);
+      const StepLoads L = begin_step(slot * CFG::STAGE_BYTES);
 #pragma unroll
       for (int j = 0; j < LA + LB; ++j) issue_one(L, j);
       end_step();
@@ -530,7 +539,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     wait_vmcnt<(STAGES - 2) * (LA + LB)>();
     __builtin_amdgcn_s_barrier();
     Frags<CFG> fr[2];
-    load_frags(fr[0], 0, 0);
+    if constexpr (!PINGPONG) load_frags(fr[0], 0, 0);
 
     // ---- main loop ----------------------------------------------------------------------------
     // Invariant at the top of step s: the operands of step s are in LDS and visible to all waves,
@@ -541,6 +550,79 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     // eight-wave tile would spill and keeps the ring position in a register.
     constexpr int RING_UNROLL = (NW == 4) ? STAGES : 1;
     int s = 0, ring_pos = 0;
+    if constexpr (PINGPONG) {
+      // Eight waves, two per SIMD: waves 0-3 and waves 4-7 run half a step apart.  A step is a
+      // memory phase (all fragment reads of the step, then the direct-to-LDS loads that refill the
+      // slot of the previous step) and a compute phase (nothing but MFMAs), each closed by a
+      // workgroup barrier, so that on every SIMD one wave feeds the matrix pipe while the other
+      // one has the LDS and memory ports to itself.
+      static_assert(KS <= 2, "one fragment set per k-slice");
+      const bool late = wave >= 4;
+      if (late) __builtin_amdgcn_s_barrier();
+      // The loader position of the common case - a whole K step inside one source - is carried in
+      // scalar registers that advance by constants, and its loads need no per-lane k test; partial
+      // steps, source changes and the empty steps past the end take the general path.
+      const unsigned b_inc = __builtin_amdgcn_readfirstlane(
+          CFG::B_KCONTIG ? (unsigned)(BK * ES) : (unsigned)((long long)BK * p.s_bk * ES));
+      unsigned a_so = 0, b_so = 0;
+      int k_left = 0;
+      auto resync = [&]() {
+        a_so = (unsigned)(i_kb * BK * ES);
+        const long long kglob = (long long)i_src * klocal + (long long)i_kb * BK;
+        b_so = __builtin_amdgcn_readfirstlane(
+            CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
+        k_left = i_step < nsteps ? klocal - i_kb * BK : 0;
+      };
+      resync();
+      unsigned rd = 0;                                    // byte offset of the slot this step reads
+      unsigned wr = (STAGES - 1) * CFG::STAGE_BYTES;      // ... and of the slot it refills
+      const unsigned wr_wave = smem_base + wave * kDmaBytes;
+      for (; s < nsteps; ++s) {
+        // Fragment reads first: they start at once, and the direct-to-LDS loads (which the address
+        // unit accepts only one wave at a time) queue up behind them instead of in front.
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) load_frags(fr[kk], rd, kk);
+        __builtin_amdgcn_sched_barrier(0);
+        if (k_left >= BK) {
+#pragma unroll
+          for (int j = 0; j < LA; ++j) dma16(ra, wr_wave + wr + j * NW * kDmaBytes, a_voff[j], a_so);
+#pragma unroll
+          for (int i = 0; i < LB; ++i)
+            dma16(rb, wr_wave + wr + CFG::A_BYTES + i * NW * kDmaBytes, b_voff[i], b_so);
+        } else {
+          const StepLoads L = begin_step(wr);
+#pragma unroll
+          for (int j = 0; j < LA + LB; ++j) issue_one(L, j);
+        }
+        end_step();
+        if (i_kb == 0) {
+          resync();
+        } else {
+          a_so += BK * ES;
+          b_so += b_inc;
+          k_left -= BK;
+        }
+        // Own fragment reads done (the slot may be refilled two barriers from here) and own loads
+        // of step s+1 landed.
+        wait_vmcnt_lgkm0<(STAGES - 2) * (LA + LB)>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+              acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        rd = rd + CFG::STAGE_BYTES == CFG::RING_BYTES ? 0 : rd + CFG::STAGE_BYTES;
+        wr = wr + CFG::STAGE_BYTES == CFG::RING_BYTES ? 0 : wr + CFG::STAGE_BYTES;
+      }
+      if (!late) __builtin_amdgcn_s_barrier();
+    } else
     while (s < nsteps) {
 #pragma unroll
     for (int u = 0; u < RING_UNROLL; ++u) {
@@ -553,16 +635,16 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       __builtin_amdgcn_s_barrier();             // everyone's have; everyone is past step s-1
       int pslot = slot + STAGES - 1;
       if (pslot >= STAGES) pslot -= STAGES;
-      const StepLoads L = begin_step(pslot);  // refills the slot the previous step used
+      const StepLoads L = begin_step(pslot * CFG::STAGE_BYTES);  // refills the slot the previous step used
       const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
       constexpr int NSLOT = KS * MB;          // MFMA groups of a step; the loads are spread over them
       constexpr int NLOAD = LA + LB;
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk) {
         if (kk + 1 < KS)
-          load_frags(fr[(kk + 1) & 1], slot, kk + 1);
+          load_frags(fr[(kk + 1) & 1], slot * CFG::STAGE_BYTES, kk + 1);
         else
-          load_frags(fr[(kk + 1) & 1], nslot, 0);
+          load_frags(fr[(kk + 1) & 1], nslot * CFG::STAGE_BYTES, 0);
         const Frags<CFG>& f = fr[kk & 1];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
