@@ -400,9 +400,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   }
 
   // Read the fragments of k-slice kk of ring slot `slot`.
-  auto load_frags = [&](Frags<CFG>& f, int slot_off, int kk) {  // slot_off: byte offset of the ring slot
-    const char* sa = smem + slot_off;
-    const char* sb = sa + CFG::A_BYTES;
+  auto load_frags_b = [&](Frags<CFG>& f, int slot_off, int kk) {  // slot_off: byte offset of the ring slot
+    const char* sb = smem + slot_off + CFG::A_BYTES;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if constexpr (CFG::B_KCONTIG) {
@@ -426,11 +425,17 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         f.b[nb][0] = (i32x4_t){u0.x, u0.y, u1.x, u1.y};
       }
     }
+  };
+  auto load_frags_a = [&](Frags<CFG>& f, int slot_off, int kk, int mb) {
+    const char* sa = smem + slot_off;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int h = 0; h < NFRAG; ++h)
+      f.a[mb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sa + fa_off[kk][h] + mb * 32 * CFG::RBA);
+  };
+  auto load_frags = [&](Frags<CFG>& f, int slot_off, int kk) {
+    load_frags_b(f, slot_off, kk);
 #pragma unroll
-      for (int h = 0; h < NFRAG; ++h)
-        f.a[mb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sa + fa_off[kk][h] + mb * 32 * CFG::RBA);
+    for (int mb = 0; mb < MB; ++mb) load_frags_a(f, slot_off, kk, mb);
   };
 
   const int total_tiles = p.tiles_m * p.tiles_n;
@@ -534,9 +539,12 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         for (int i = 0; i < 16; ++i) acc.v[mb][nb][i] = 0.f;
 
     // ---- prologue: fill STAGES-1 ring slots, wait for the first ----------------------------------
+    // The two-group loop reads a slot in both of its phases and refills it one step later than the
+    // single-group loop, so it keeps one step less in flight.
+    constexpr int AHEAD = PINGPONG ? STAGES - 2 : STAGES - 1;  // K steps issued before the loop starts
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s);
-    wait_vmcnt<(STAGES - 2) * (LA + LB)>();
+    for (int s = 0; s < AHEAD; ++s) issue(s);
+    wait_vmcnt<(AHEAD - 1) * (LA + LB)>();
     __builtin_amdgcn_s_barrier();
     Frags<CFG> fr[2];
     if constexpr (!PINGPONG) load_frags(fr[0], 0, 0);
@@ -575,13 +583,23 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       };
       resync();
       unsigned rd = 0;                                    // byte offset of the slot this step reads
-      unsigned wr = (STAGES - 1) * CFG::STAGE_BYTES;      // ... and of the slot it refills
+      unsigned wr = AHEAD * CFG::STAGE_BYTES;             // ... and of the slot it refills
       const unsigned wr_wave = smem_base + wave * kDmaBytes;
+      // The fragments of the first half of a step's MFMAs are read in the memory phase, those of the
+      // second half between the MFMAs of the first (LDS reads issue in the shadow of an MFMA;
+      // direct-to-LDS loads do not, a wave takes some 80 cycles to get one accepted).
+      constexpr int NMFMA = KS * MB * NB;
+      constexpr bool SPLIT_K = KS >= 2;                    // halves split by k-slice, else by row block
+      static_assert(KS == 1 || KS == 2, "fragment sets of the two-group loop");
+      static_assert(MB % 2 == 0, "row blocks split in two halves");
       for (; s < nsteps; ++s) {
-        // Fragment reads first: they start at once, and the direct-to-LDS loads (which the address
-        // unit accepts only one wave at a time) queue up behind them instead of in front.
+        if constexpr (SPLIT_K) {
+          load_frags(fr[0], rd, 0);
+        } else {
+          load_frags_b(fr[0], rd, 0);
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) load_frags(fr[kk], rd, kk);
+          for (int mb = 0; mb < MB / 2; ++mb) load_frags_a(fr[0], rd, 0, mb);
+        }
         __builtin_amdgcn_sched_barrier(0);
         if (k_left >= BK) {
 #pragma unroll
@@ -602,19 +620,29 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           b_so += b_inc;
           k_left -= BK;
         }
-        // Own fragment reads done (the slot may be refilled two barriers from here) and own loads
-        // of step s+1 landed.
-        wait_vmcnt_lgkm0<(STAGES - 2) * (LA + LB)>();
+        // Own early fragment reads done and own loads of step s+1 landed.
+        wait_vmcnt_lgkm0<(AHEAD - 1) * (LA + LB)>();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
+        // First half of the MFMAs, one late fragment read after each of the first few.
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk)
+        for (int i = 0; i < NMFMA / 2; ++i) {
+          const int kk = SPLIT_K ? 0 : 0, mb = i / NB, nb = i % NB;
+          acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
+          if constexpr (SPLIT_K) {
+            if (i == 0) load_frags_b(fr[1], rd, 1);
+            if (i >= 1 && i <= MB) load_frags_a(fr[1], rd, 1, i - 1);
+          } else {
+            if (i < MB / 2) load_frags_a(fr[0], rd, 0, MB / 2 + i);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-              acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
+        for (int i = NMFMA / 2; i < NMFMA; ++i) {
+          const int kk = SPLIT_K ? 1 : 0, mb = SPLIT_K ? (i - NMFMA / 2) / NB : i / NB, nb = i % NB;
+          acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
+        }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
