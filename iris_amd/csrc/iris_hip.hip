@@ -1171,8 +1171,13 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   }
   const int total = p.tiles_m * p.tiles_n;
   const int cap = cu_count * CFG::WG_PER_CU;
+  // A multiple of the XCD count keeps the XCD mapping exact.  Rounded up when the tiles fit in one
+  // round (the surplus workgroups find no tile and leave), so that no tile waits for a second round.
   int grid = total < cap ? total : cap;
-  if (grid >= p.num_xcd) grid -= grid % p.num_xcd;  // keep the XCD mapping exact
+  if (grid % p.num_xcd) {
+    const int up = grid + p.num_xcd - grid % p.num_xcd;
+    grid = up <= cap ? up : grid - grid % p.num_xcd;
+  }
   if (grid < 1) grid = 1;
   hipLaunchKernelGGL(fused_mfma_kernel<CFG>, dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
   snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name);
