@@ -64,7 +64,7 @@ enum {
   IRIS_HIP_PATH_GENERIC = 2 /* generic kernel */
 };
 
-/* Bits set in *status by a kernel. */
+/* Codes stored to *status by a kernel. */
 enum {
   IRIS_HIP_STATUS_SPIN_TIMEOUT = 1 /* a peer flag did not become 1 within spin_limit polls */
 };
@@ -87,7 +87,8 @@ enum {
  * block_size_k is accepted for signature parity and does not change any result.
  * scale multiplies the fp32 product before the cast (use scale_a*scale_b for fp8, 1.0f otherwise).
  * spin_limit <= 0 spins without bound like the reference; > 0 gives up after that many polls of one
- * flag and ORs IRIS_HIP_STATUS_SPIN_TIMEOUT into *status (status may be NULL).
+ * flag and stores IRIS_HIP_STATUS_SPIN_TIMEOUT to *status (status may be NULL; device memory or
+ * device-visible pinned host memory).
  */
 int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
                                int64_t M, int64_t N, int64_t K,

@@ -150,7 +150,9 @@ __device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, in
     long long polls = 0;
     while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != 1) {
       if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
-        if (p.status) atomicOr(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT);
+        // A plain system-scope store (one status code, every writer stores the same word): the word
+        // may live in pinned host memory.
+        if (p.status) __hip_atomic_store(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         break;
       }
       __builtin_amdgcn_s_sleep(8);

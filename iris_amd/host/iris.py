@@ -84,7 +84,13 @@ class Iris:
         self._cu_count = None
         # Flag-wait bound handed to the kernels (polls per flag; <= 0 waits forever as the reference).
         self.spin_limit = int(os.environ.get("IRIS_SPIN_LIMIT", str(1 << 22)))
-        self._status = torch.zeros(1, dtype=torch.int32, device=self.heap.device)
+        # Status word the kernels write on a flag-wait timeout.  With a GPU it lives in pinned host
+        # memory (device-visible at the same address), so that every barrier can read it without a
+        # device-to-host copy.
+        if self.heap.device.type == "cuda":
+            self._status = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        else:
+            self._status = torch.zeros(1, dtype=torch.int32, device=self.heap.device)
         # One GPU standing in for all ranks: when set, the fused operators' preambles mark the other
         # ranks as finished (flags raised, aux zeroed) so that a launch does not wait for them.
         self.stand_in_peers = os.environ.get("IRIS_STAND_IN_PEERS", "0") not in ("", "0")
@@ -261,7 +267,7 @@ class Iris:
 
     def check_status(self):
         """Raise RuntimeError if a kernel set a status bit since the last check (needs a sync first)."""
-        status = int(self._status.item())
+        status = int(self._status[0])
         if status:
             self._status.zero_()
             raise RuntimeError(
