@@ -548,7 +548,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     for (int s = 0; s < AHEAD; ++s) issue(s);
     wait_vmcnt<(AHEAD - 1) * (LA + LB)>();
     __builtin_amdgcn_s_barrier();
-    Frags<CFG> fr[2];
+    Frags<CFG> fr[KS < 2 ? 2 : KS];  // one set per k-slice (two for the loops that double-buffer)
     if constexpr (!PINGPONG) load_frags(fr[0], 0, 0);
 
     // ---- main loop ----------------------------------------------------------------------------
@@ -566,7 +566,6 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // slot of the previous step) and a compute phase (nothing but MFMAs), each closed by a
       // workgroup barrier, so that on every SIMD one wave feeds the matrix pipe while the other
       // one has the LDS and memory ports to itself.
-      static_assert(KS <= 2, "one fragment set per k-slice");
       const bool late = wave >= 4;
       if (late) __builtin_amdgcn_s_barrier();
       // The loader position of the common case - a whole K step inside one source - is carried in
@@ -592,11 +591,26 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // direct-to-LDS loads do not, a wave takes some 80 cycles to get one accepted).
       constexpr int NMFMA = KS * MB * NB;
       constexpr bool SPLIT_K = KS >= 2;                    // halves split by k-slice, else by row block
-      static_assert(KS == 1 || KS == 2, "fragment sets of the two-group loop");
+      static_assert(KS == 1 || KS % 2 == 0, "k-slices split in two halves");
       static_assert(MB % 2 == 0, "row blocks split in two halves");
+      // Late fragment reads, in pieces: per late k-slice the B fragments, then one row block of A each;
+      // with a single slice the upper row blocks of A.
+      constexpr int LATE_PIECES = SPLIT_K ? (KS / 2) * (1 + MB) : MB / 2;
+      auto late_piece = [&](int pc) {
+        if constexpr (SPLIT_K) {
+          const int kk = KS / 2 + pc / (1 + MB), q = pc % (1 + MB);
+          if (q == 0)
+            load_frags_b(fr[kk], rd, kk);
+          else
+            load_frags_a(fr[kk], rd, kk, q - 1);
+        } else {
+          load_frags_a(fr[0], rd, 0, MB / 2 + pc);
+        }
+      };
       for (; s < nsteps; ++s) {
         if constexpr (SPLIT_K) {
-          load_frags(fr[0], rd, 0);
+#pragma unroll
+          for (int kk = 0; kk < KS / 2; ++kk) load_frags(fr[kk], rd, kk);
         } else {
           load_frags_b(fr[0], rd, 0);
 #pragma unroll
@@ -627,22 +641,19 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        // First half of the MFMAs, one late fragment read after each of the first few.
+        // First half of the MFMAs with the late fragment reads spread between them.
 #pragma unroll
         for (int i = 0; i < NMFMA / 2; ++i) {
-          const int kk = SPLIT_K ? 0 : 0, mb = i / NB, nb = i % NB;
+          const int kk = i / (MB * NB), mb = (i / NB) % MB, nb = i % NB;  // one slice: mb < MB/2 here
           acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
-          if constexpr (SPLIT_K) {
-            if (i == 0) load_frags_b(fr[1], rd, 1);
-            if (i >= 1 && i <= MB) load_frags_a(fr[1], rd, 1, i - 1);
-          } else {
-            if (i < MB / 2) load_frags_a(fr[0], rd, 0, MB / 2 + i);
-          }
+#pragma unroll
+          for (int pc = 0; pc < LATE_PIECES; ++pc)
+            if (pc * (NMFMA / 2) / LATE_PIECES == i) late_piece(pc);
           __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int i = NMFMA / 2; i < NMFMA; ++i) {
-          const int kk = SPLIT_K ? 1 : 0, mb = SPLIT_K ? (i - NMFMA / 2) / NB : i / NB, nb = i % NB;
+          const int kk = i / (MB * NB), mb = (i / NB) % MB, nb = i % NB;
           acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
         }
         __builtin_amdgcn_sched_barrier(0);
