@@ -486,6 +486,27 @@ def test_ragged_shapes_mfma(M, N, K, variant):
         assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
 
 
+# Tile counts that are not a multiple of the eight XCDs and fit in one round: the launch grid is rounded
+# up and the surplus workgroups must find no tile (23 tiles of 64x128 and of 128x128, 27 of 128x128,
+# 140 of 256x256).
+@pytest.mark.parametrize("M,N,K,tile", [(32, 2880, 64, "64x128"), (96, 2880, 64, "128x128"),
+                                        (384, 1152, 96, "128x128"), (2560, 3584, 64, "256x256")])
+def test_tile_counts_off_the_xcd_multiple(M, N, K, tile):
+    W, rank, dtype = 2, 1, torch.float16
+    ctx = _ctx(W, rank, heap=1 << 27)
+    A, B = randint_cpu((M, K), 52, dtype), randint_cpu((K, N), 53, dtype)
+    peers = [randn_cpu((M, N), 620 + r, dtype) for r in range(W)]
+    cfg = iris.FusedConfig(block_size_m=32, block_size_n=64, block_size_k=8, all_reduce_variant="two_shot")
+    dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg, path="mfma")
+    assert kernel.startswith(f"mfma_f16_{tile}"), kernel
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, 32, 64, "two_shot", "fp32")
+    assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], "aux")
+    assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+    got = slot_copies(ctx, dC)
+    for r in range(W):
+        assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
+
+
 @pytest.mark.parametrize("M,N,K", [(200, 272, 80), (1, 1024, 256), (520, 144, 1008)])
 def test_ragged_shapes_mfma_fp8(M, N, K):
     W, rank = 4, 1
