@@ -176,11 +176,12 @@ def test_ragged_shapes_generic(M, N, K):
     assert torch.all(ws.locks.cpu() == 1)
 
 
-def test_transposed_b_and_strided_views():
-    """B handed over as the transpose of an (N, K) tensor (K-contiguous) takes the MFMA path too."""
-    ctx = _ctx(1)
+@pytest.mark.parametrize("M,N,K", [(256, 384, 128), (3072, 3072, 200)])
+def test_transposed_b_and_strided_views(M, N, K):
+    """B handed over as the transpose of an (N, K) tensor (K-contiguous) takes the MFMA path too
+    (128x128 tiles for the first shape, 256x256 for the second)."""
+    ctx = _ctx(1, heap=1 << 27)
     dtype = torch.bfloat16
-    M, N, K = 256, 384, 128
     A, Bt = randint_cpu((M, K), 8, dtype), randint_cpu((N, K), 9, dtype)
     dA, dBt = heap_tensor(ctx, A), heap_tensor(ctx, Bt)
     dC = ctx.zeros((M, N), dtype=dtype)
@@ -264,6 +265,29 @@ def test_all_gather_matmul_columns(path, M, K_local, N, W):
     ops.all_gather_matmul(ctx, out, dA, dB, config=cfg, kernel_path=path)
     assert _lib.last_kernel().startswith(path)
     assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B), _lib.last_kernel())
+
+
+# The 256x256 tile (two wave groups half a K step apart) gathering along K: the A source changes in the
+# middle of the load pipeline; K_local = 80 ends every source with a partial K step, 1 with an almost
+# empty one.
+@pytest.mark.parametrize("K_local,W", [(96, 4), (80, 3), (32, 8), (1, 2)])
+def test_all_gather_matmul_columns_big_tile(K_local, W):
+    M = N = 3072
+    dtype, rank = torch.bfloat16, W - 1
+    ctx = _ctx(W, rank, heap=1 << 27)
+    shards = [randint_cpu((M, K_local), 42 + r, dtype) for r in range(W)]
+    B = randint_cpu((W * K_local, N), 123, dtype)
+    ok_mfma = K_local % 8 == 0
+    dA = ctx.zeros((M, K_local), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    out = ctx.zeros((M, N), dtype=dtype)
+    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=1)
+    ops.all_gather_matmul(ctx, out, dA, dB, config=cfg)
+    kernel = _lib.last_kernel()
+    assert kernel.startswith("mfma_bf16_256x256" if ok_mfma else "generic"), kernel
+    assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B), kernel)
 
 
 def test_all_gather_matmul_rows_and_bias():
