@@ -357,6 +357,25 @@ def test_matmul_all_gather(path, dtype, M, N, K):
             assert_bits_equal(got, exp[r], f"{_lib.last_kernel()} rank {rank} slot {r}")
 
 
+def test_matmul_all_gather_big_tile():
+    """Enough rows per rank for the 256x256 tile (16 x 9 tiles), row bias, two slots."""
+    W, rank, dtype = 2, 1, torch.bfloat16
+    M_local, N, K = 4096, 2304, 72
+    B = randint_cpu((K, N), 77, dtype, -2, 3)
+    A = randint_cpu((M_local, K), 81, dtype, -2, 3)
+    bias = randint_cpu((M_local,), 90, dtype, -4, 5)
+    ctx = _ctx(W, rank, heap=1 << 27)
+    dA, dB, dbias = heap_tensor(ctx, A), heap_tensor(ctx, B), heap_tensor(ctx, bias)
+    out = ctx.zeros((W * M_local, N), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(out, r).zero_()
+    ctx.ops.matmul_all_gather(out, dA, dB, bias=dbias, config=iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=8))
+    assert _lib.last_kernel().startswith("mfma_bf16_256x256"), _lib.last_kernel()
+    exp = oracle.matmul_all_gather(A, B, rank, W, bias=bias)
+    for r, got in enumerate(slot_copies(ctx, out)):
+        assert_bits_equal(got, exp[r], f"slot {r}")
+
+
 @pytest.mark.parametrize("path", ["mfma", "generic"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_all_reduce_atomic(path, dtype):
