@@ -840,9 +840,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
         constexpr bool NT = decltype(nt_tag)::value;  // peers' tiles and C bypass the caches' keep policy
         constexpr int NPV = NP > 0 ? NP : 1;
-        constexpr int G = NP >= 4 ? 2 : 4;           // passes whose loads are issued together
+        // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
+        // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
+        // at a time also with seven peers, and groups below the last row of the matrix are skipped.
+        constexpr int G = (NP >= 4 && NW == 8) ? 2 : 4;
         static_assert(PASSES % G == 0, "pass grouping");
         for (int pg = 0; pg < PASSES; pg += G) {
+          if (m0 + pg * RPP >= p.M) break;
           bool active[G];
           long long eoff[G];
           int owner[G];
