@@ -5,15 +5,20 @@
 The library lands in iris_amd/lib/ next to the package so that it travels with the source tree.
 """
 
+import concurrent.futures
 import os
 import shutil
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-SOURCES = [os.path.join(HERE, "iris_hip.hip"), os.path.join(HERE, "iris_ccl.hip")]
-HEADERS = [os.path.join(HERE, h) for h in ("layout.h", "device_util.h", "host_common.h")] + [
+# One translation unit per input type of the MFMA kernel (they hold most of the compile time and are
+# compiled side by side), the entry points with the generic kernel, and the stand-alone collectives.
+SOURCES = [os.path.join(HERE, f) for f in (
+    "iris_hip.hip", "iris_hip_mfma_bf16.hip", "iris_hip_mfma_f16.hip", "iris_hip_mfma_fp8.hip", "iris_ccl.hip")]
+HEADERS = [os.path.join(HERE, h) for h in ("fused_kernel.h", "layout.h", "device_util.h", "host_common.h")] + [
     os.path.join(ROOT, "include", "iris_hip.h")]
 OUTPUT = os.path.join(os.path.dirname(HERE), "lib", "libiris_hip.so")
 
@@ -22,7 +27,6 @@ FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # Keep hipcc from forming packed fp32 instructions out of scalar float code.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unknown-warning-option",
@@ -38,14 +42,7 @@ def up_to_date():
     return all(os.path.getmtime(f) <= built for f in SOURCES + HEADERS + [os.path.abspath(__file__)])
 
 
-def build(force=True, verbose=True):
-    """Compile the library.  With force=False an up-to-date library is left alone."""
-    if not force and up_to_date():
-        return OUTPUT
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    os.makedirs(os.path.dirname(OUTPUT), exist_ok=True)
-    tmp = OUTPUT + ".tmp"
-    cmd = [hipcc] + FLAGS + ["-o", tmp] + SOURCES
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -53,10 +50,27 @@ def build(force=True, verbose=True):
     noise = "is not a recognized feature for this target"
     out = "\n".join(l for l in proc.stdout.splitlines() if noise not in l)
     if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
+        raise RuntimeError(f"hipcc failed ({proc.returncode}): {' '.join(cmd)}\n{out}")
     if verbose and out.strip():
         print(out)
-    os.replace(tmp, OUTPUT)
+
+
+def build(force=True, verbose=True):
+    """Compile the library.  With force=False an up-to-date library is left alone."""
+    if not force and up_to_date():
+        return OUTPUT
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    os.makedirs(os.path.dirname(OUTPUT), exist_ok=True)
+    with tempfile.TemporaryDirectory(prefix="iris_hip_build_") as tmpdir:
+        objects = [os.path.join(tmpdir, os.path.splitext(os.path.basename(src))[0] + ".o") for src in SOURCES]
+        with concurrent.futures.ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
+            jobs = [pool.submit(_run, [hipcc] + FLAGS + ["-c", "-o", obj, src], verbose)
+                    for src, obj in zip(SOURCES, objects)]
+            for job in jobs:
+                job.result()
+        tmp = OUTPUT + ".tmp"
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp] + objects, verbose)
+        os.replace(tmp, OUTPUT)
     return OUTPUT
 
 

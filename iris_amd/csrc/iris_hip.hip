@@ -1,7 +1,8 @@
 // libiris_hip: gfx950 (MI355X) kernels for the rank-local compute of the fused GEMM+collective
 // operators, and the C ABI declared in include/iris_hip.h.
 //
-// Two kernels implement every operator:
+// Two kernels implement every operator (the first lives in fused_kernel.h and is compiled in the
+// iris_hip_mfma_<type>.hip translation units, the second and the entry points are in this file):
 //
 //  * fused_mfma_kernel  - persistent tiled GEMM on the 32x32 MFMA blocks of CDNA4.  Operand tiles
 //    travel HBM -> LDS with 16-byte direct-to-LDS buffer loads into a ring of STAGES buffers
@@ -31,912 +32,7 @@
 
 #include <type_traits>
 
-#include "iris_hip.h"
-#include "layout.h"
-#include "device_util.h"
-#include "host_common.h"
-
-using namespace iris_layout;
-
-#define LDS_AS __attribute__((address_space(3)))
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(16))) float f32x16_t;
-typedef __attribute__((ext_vector_type(2))) int i32x2_t;
-typedef __attribute__((ext_vector_type(4))) int i32x4_t;
-typedef __attribute__((ext_vector_type(8))) int i32x8_t;
-typedef __attribute__((ext_vector_type(4))) short i16x4_t;
-typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
-typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
-
-enum { EPI_STORE = 0, EPI_ONE_SHOT = 1, EPI_TWO_SHOT = 2, EPI_REDUCE_SCATTER = 3, EPI_ALL_GATHER = 4, EPI_ATOMIC = 5 };
-
-// Epilogues that publish aux + flags and then reduce over the slots.
-__host__ __device__ inline bool epi_has_flags(int epi) { return epi == EPI_ONE_SHOT || epi == EPI_TWO_SHOT || epi == EPI_REDUCE_SCATTER; }
-enum { GATHER_NONE = 0, GATHER_K = 1, GATHER_M = 2 };
-
-struct FusedParams {
-  const char* A;
-  const char* B;
-  char* C;
-  char* aux;
-  int* locks;
-  const char* bias;
-  int M, N, K;
-  int K_local;  // K extent held by one source slot (== K unless gathered along K)
-  int M_local;  // rows held by one source slot when gathered along M
-  int gather;
-  long long s_am, s_ak, s_bk, s_bn, s_cm, s_cn, s_bias;  // element strides
-  const long long* heap_bases;
-  int rank, world;
-  int flag_bm, flag_bn;
-  int epi;
-  int acc_mode;
-  int all_owners;
-  int sum_peers;
-  int bias_dtype;
-  float scale;
-  long long spin_limit;
-  int* status;
-  int tiles_m, tiles_n, group_m, num_xcd;
-  int row_offset;  // all-gather: first row of this rank's block in the gathered output
-  int stream_peers;  // phase 2 reads the peers' tiles and writes C with non-temporal accesses
-};
-
-// ------------------------------------------------------------------------------------------------
-// Small device helpers
-// ------------------------------------------------------------------------------------------------
-
-__device__ __forceinline__ int owner_of(int epi, int t, int total, int world, int rank) {
-  if (epi == EPI_TWO_SHOT) return owner_interleaved(t, world);
-  if (epi == EPI_REDUCE_SCATTER) return owner_contiguous(t, total, world);
-  return rank;
-}
-
-// Raise the flags of the flag tiles covered by the macro tile at (m0, n0) of KM x KN elements.
-// Must be called by every thread of the workgroup after the workgroup's aux stores have completed
-// (vmcnt(0)) and a workgroup barrier.
-// WRITTEN_THROUGH = false: the aux stores were ordinary stores (dirty lines in L2), so the flag is
-//   raised with system-scope release, which writes the L2 back first.
-// WRITTEN_THROUGH = true: the aux stores were system-scope write-through stores (store16_system) that
-//   have been acknowledged, so the data is already where a peer reads it and a relaxed system-scope
-//   flag store after them is enough; this spares one whole-L2 write-back per workgroup (measured 5-11 %
-//   of the fused launch).
-template <int KM, int KN, int NT, bool WRITTEN_THROUGH>
-__device__ __forceinline__ void raise_flags(const FusedParams& p, int m0, int n0, int tid) {
-  const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
-  const int ftn = cdiv(p.N, p.flag_bn);
-  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
-  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
-  const int nfn = fn_hi - fn_lo + 1;
-  const int nft = (fm_hi - fm_lo + 1) * nfn;
-  for (int i = tid; i < nft; i += NT) {
-    const int fm = fm_lo + i / nfn, fn = fn_lo + i % nfn;
-    int* flag = p.locks + (fm * ftn + fn);
-    const int needed = macro_tiles_over_flag_tile(fm, fn, p.flag_bm, p.flag_bn, KM, KN, p.M, p.N);
-    bool last = true;
-    if (needed > 1) {
-      // Arrivals are counted in steps of 2 so that the flag never reads 1 before the last one.
-      int old = WRITTEN_THROUGH ? __hip_atomic_fetch_add(flag, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
-                                : __hip_atomic_fetch_add(flag, 2, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_SYSTEM);
-      last = ((old >> 1) + 1) == needed;
-    }
-    if (last) {
-      if (WRITTEN_THROUGH) __hip_atomic_exchange(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      else __hip_atomic_exchange(flag, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
-  }
-}
-
-// Wait until the peers' flags of every flag tile this workgroup reduces are 1.
-template <int KM, int KN, int NT>
-__device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, int n0, int tid) {
-  const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
-  const int ftn = cdiv(p.N, p.flag_bn);
-  const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
-  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
-  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
-  const int nfn = fn_hi - fn_lo + 1;
-  const int nft = (fm_hi - fm_lo + 1) * nfn;
-  const int items = nft * p.world;
-  for (int i = tid; i < items; i += NT) {
-    const int r = i % p.world;
-    const int f = i / p.world;
-    if (r == p.rank) continue;
-    const int t = (fm_lo + f / nfn) * ftn + fn_lo + f % nfn;
-    if (!p.all_owners && owner_of(p.epi, t, ftotal, p.world, p.rank) != p.rank) continue;
-    const int* flag = (const int*)slot_ptr(p.heap_bases, p.locks + t, p.rank, r);
-    long long polls = 0;
-    while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != 1) {
-      if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
-        // A plain system-scope store (one status code, every writer stores the same word): the word
-        // may live in pinned host memory.
-        if (p.status) __hip_atomic_store(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
-    }
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
-// MFMA kernel configuration
-// ------------------------------------------------------------------------------------------------
-enum { IN_BF16 = 0, IN_F16 = 1, IN_FP8 = 2 };
-
-template <int IN_, int BM_, int BN_, int BK_, int WM_, int WN_, int STAGES_, bool B_KCONTIG_>
-struct MfmaCfg {
-  static constexpr int IN = IN_;
-  static constexpr int ES = (IN_ == IN_FP8) ? 1 : 2;
-  static constexpr int CE = kChunkBytes / ES;           // elements per 16-byte chunk
-  static constexpr int KM = (IN_ == IN_FP8) ? 64 : 16;  // k per MFMA
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_;
-  static constexpr bool B_KCONTIG = B_KCONTIG_;
-  static constexpr int WM = WM_, WN = WN_, NW = WM_ * WN_, NT = 64 * NW;
-  static constexpr int TM = BM / WM, TN = BN / WN;  // per-wave block
-  static constexpr int MB = TM / 32, NB = TN / 32;  // 32x32 MFMA blocks per wave
-  static constexpr int KSLICES = BK / KM;
-  static constexpr int NFRAG = (IN_ == IN_FP8) ? 2 : 1;   // 16-byte pieces per operand fragment
-  static constexpr int RBA = BK * ES;                        // bytes per A tile row
-  static constexpr int RBB = B_KCONTIG ? BK * ES : BN * ES;  // bytes per B tile row
-  static constexpr int A_BYTES = BM * RBA;
-  static constexpr int B_BYTES = B_KCONTIG ? BN * RBB : BK * RBB;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LA = A_BYTES / kDmaBytes / NW;  // direct-to-LDS loads per thread per K step
-  static constexpr int LB = B_BYTES / kDmaBytes / NW;
-  static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
-  // Epilogue staging: the whole output tile in 16-bit elements, rows padded by 16 bytes so that
-  // the accumulator-layout writes (one row per lane) spread over the LDS banks.
-  static constexpr int TROW = BN * 2 + 16;
-  static constexpr int TILE_BYTES = BM * TROW;
-  static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES;
-  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
-  // Four-wave tiles whose ring fits twice into a CU's LDS run two workgroups per CU, so that the
-  // memory round trips of one workgroup's epilogue hide behind the other's K loop.
-  static constexpr int WG_PER_CU = (NW == 4 && SMEM_BYTES <= 80 * 1024) ? 2 : 1;
-  static constexpr int WAVES_PER_SIMD = WG_PER_CU * NW / 4;
-  static_assert(NT % (BN / 8) == 0 && BM % (NT / (BN / 8)) == 0, "epilogue pass shape");
-  static_assert(A_BYTES % (kDmaBytes * NW) == 0 && B_BYTES % (kDmaBytes * NW) == 0, "tile/loader mismatch");
-  static_assert(BK % KM == 0 && TM % 32 == 0 && TN % 32 == 0, "tile/MFMA mismatch");
-  static_assert(STAGES >= 3, "the ring needs at least three slots");
-  static_assert((STAGES - 2) * (LA + LB) <= 63, "vmcnt field too small for this prefetch depth");
-};
-
-template <int IN>
-struct OutOf { using type = OutBF16; };
-template <>
-struct OutOf<IN_F16> { using type = OutF16; };
-
-// s_waitcnt vmcnt(n) with the other counters left unconstrained (gfx9 encoding).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
-}
-
-// The same with lgkmcnt(0): every LDS read of this wave has returned as well.
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_lgkm0() {
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4));
-}
-
-constexpr unsigned kInvalidOffset = 0x80000000u;
-
-// Buffer resource words for a raw buffer (stride 0) over [base, base + 2^31).  Bounds are enforced
-// per lane by the callers: an invalid lane presents offset 0x80000000, which is past num_records
-// and therefore loads zero.
-__device__ __forceinline__ i32x4_t make_rsrc_words(unsigned long long b) {
-  i32x4_t r;
-  r.x = __builtin_amdgcn_readfirstlane((int)(unsigned)b);
-  r.y = __builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
-  r.z = 0x7FFFFFFF;
-  r.w = 0x00020000;
-  return r;
-}
-
-// One wave-wide 16-byte direct-to-LDS load: lane l deposits global bytes [voff + soff, +16) of the
-// buffer at LDS address lds_base + 16*l.  Written as inline assembly so that the compiler's
-// wait-count pass does not serialise LDS reads behind loads that target other ring slots; the
-// kernel orders them itself with wait_vmcnt() and workgroup barriers.
-__device__ __forceinline__ void dma16(i32x4_t rsrc, unsigned lds_base, unsigned voff, unsigned soff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-               : "memory");
-}
-
-// 16-byte store that is written through to memory at system scope (sc0 sc1): once vmcnt reports it
-// done, every agent that reads the address with a coherent load sees it, without an L2 write-back.
-__device__ __forceinline__ void store16_system(char* p, u32x4_t v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
-}
-
-// Read one accumulator register.  The "a" constraint keeps the MFMA results in the accumulation
-// registers until the epilogue consumes them, instead of copying all of them to VGPRs at once.
-__device__ __forceinline__ float acc_read(float a) {
-  float v;
-  asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-  return v;
-}
-
-__device__ __forceinline__ unsigned lds_address(const void* p) {
-  return (unsigned)(unsigned long long)(LDS_AS const char*)p;
-}
-
-template <class CFG>
-struct MfmaAcc {
-  f32x16_t v[CFG::MB][CFG::NB];
-};
-
-// Operand fragments of one k-slice for a wave's block.
-template <class CFG>
-struct Frags {
-  i32x4_t a[CFG::MB][CFG::NFRAG];
-  i32x4_t b[CFG::NB][CFG::NFRAG];
-};
-
-// One 32x32 MFMA with the operands in the order (B fragment, A fragment): the accumulator then
-// holds D[n][m], i.e. each lane owns 4 consecutive n for one m.
-template <int IN, int NF>
-__device__ __forceinline__ f32x16_t mfma_block(const i32x4_t (&a)[NF], const i32x4_t (&b)[NF], f32x16_t c) {
-  if constexpr (IN == IN_BF16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, b[0]),
-                                                   __builtin_bit_cast(bf16x8_t, a[0]), c, 0, 0, 0);
-  } else if constexpr (IN == IN_F16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, b[0]),
-                                                  __builtin_bit_cast(f16x8_t, a[0]), c, 0, 0, 0);
-  } else {
-    i32x8_t av, bv;
-    av.lo = a[0]; av.hi = a[1];
-    bv.lo = b[0]; bv.hi = b[1];
-    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled
-    // instruction (v_mfma_f32_32x32x64_f8f6f4).
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 0, 0, 0, 0, 0, 0);
-  }
-}
-
-constexpr int kMaxCachedSlots = 8;  // heap bases kept in registers; larger worlds re-load them
-
-// ------------------------------------------------------------------------------------------------
-// MFMA kernel
-// ------------------------------------------------------------------------------------------------
-// ONE_ROUND: the launch has a workgroup for every tile, so a workgroup handles at most one.  The
-// tile loop is then known to run once, which lets the compiler drop everything it otherwise carries
-// from tile to tile (measured: 1.2 us of a 9 us launch on decode-sized problems).
-template <class CFG, bool ONE_ROUND>
-__global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kernel(const FusedParams p) {
-  using Out = typename OutOf<CFG::IN>::type;
-  using ATile = RowTile<CFG::RBA>;
-  constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
-  constexpr int MB = CFG::MB, NB = CFG::NB, TM = CFG::TM, TN = CFG::TN, NW = CFG::NW, NT = CFG::NT;
-  constexpr bool PINGPONG = CFG::NW == 8;
-  constexpr int STAGES = CFG::STAGES, LA = CFG::LA, LB = CFG::LB, NFRAG = CFG::NFRAG, KS = CFG::KSLICES;
-
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / CFG::WN, wn = wave % CFG::WN;
-
-  // Heap bases of the first slots, read once (scalar loads) before the kernel stores anything.
-  unsigned long long hb[kMaxCachedSlots];
-#pragma unroll
-  for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (p.heap_bases && r < p.world) ? (unsigned long long)p.heap_bases[r] : 0ull;
-  const unsigned long long hb_own = p.heap_bases ? (unsigned long long)p.heap_bases[p.rank] : 0ull;
-  auto heap_base = [&](int r) -> unsigned long long {
-    unsigned long long v = 0;
-    if (r < kMaxCachedSlots) {
-#pragma unroll
-      for (int q = 0; q < kMaxCachedSlots; ++q) v = (r == q) ? hb[q] : v;
-    } else {
-      v = (unsigned long long)p.heap_bases[r];
-    }
-    return v;
-  };
-  // Address in slot r of own-slot address `own`.
-  auto in_slot = [&](unsigned long long own, int r) -> unsigned long long { return heap_base(r) + (own - hb_own); };
-
-  // ---- loader descriptors (tile independent) ---------------------------------------------------
-  // A: row tile [BM][RBA].
-  int la_row[LA], la_k[LA];
-  unsigned la_off[LA];
-#pragma unroll
-  for (int i = 0; i < LA; ++i) {
-    int row, c;
-    ATile::from_lds((wave + i * NW) * kDmaBytes + lane * kChunkBytes, row, c);
-    la_row[i] = row;
-    la_k[i] = c * CE;
-    la_off[i] = (unsigned)(row * p.s_am * ES + c * kChunkBytes);
-  }
-  // B: col tile [BK][BN*ES] (row-major B) or row tile [BN][RBA] (B given K-contiguous).
-  int lb_row[LB], lb_col[LB];  // col tile: (k row, n element); row tile: (n row, k element)
-  unsigned lb_off[LB];
-#pragma unroll
-  for (int i = 0; i < LB; ++i) {
-    int row, c;
-    const int off = (wave + i * NW) * kDmaBytes + lane * kChunkBytes;
-    if constexpr (CFG::B_KCONTIG) {
-      RowTile<CFG::RBB>::from_lds(off, row, c);
-      lb_off[i] = (unsigned)(row * p.s_bn * ES + c * kChunkBytes);
-    } else {
-      ColTile<CFG::RBB, ES>::from_lds(off, row, c);
-      lb_off[i] = (unsigned)(row * p.s_bk * ES + c * kChunkBytes);
-    }
-    lb_row[i] = row;
-    lb_col[i] = c * CE;
-  }
-
-  // ---- fragment read offsets (relative to the slot's A / B region) -------------------------------
-  int fa_off[KS][NFRAG];
-#pragma unroll
-  for (int kk = 0; kk < KS; ++kk)
-#pragma unroll
-    for (int h = 0; h < NFRAG; ++h) {
-      const int c = (CFG::IN == IN_FP8) ? frag8_chunk(lane, kk, h) : frag16_chunk(lane, kk);
-      fa_off[kk][h] = ATile::lds_offset(wm * TM + frag16_row(lane), c);
-    }
-  // B operand: K-contiguous B reads exactly like A; row-major B uses transpose reads.
-  constexpr int NTR = (CFG::IN == IN_FP8) ? 1 : 2;  // distinct swizzles among the transpose reads
-  int fb_off[CFG::B_KCONTIG ? KS : NB][CFG::B_KCONTIG ? NFRAG : NTR];
-  if constexpr (CFG::B_KCONTIG) {
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk)
-#pragma unroll
-      for (int h = 0; h < NFRAG; ++h) {
-        const int c = (CFG::IN == IN_FP8) ? frag8_chunk(lane, kk, h) : frag16_chunk(lane, kk);
-        fb_off[kk][h] = RowTile<CFG::RBB>::lds_offset(wn * TN + frag16_row(lane), c);
-      }
-  } else {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int j = 0; j < NTR; ++j) {
-        int krow, n;
-        if constexpr (CFG::IN == IN_FP8) {
-          krow = tr8_krow(lane, 0, 0);
-          n = wn * TN + nb * 32 + tr8_ncol(lane);
-        } else {
-          krow = tr16_krow(lane, 0, j);
-          n = wn * TN + nb * 32 + tr16_ncol(lane);
-        }
-        fb_off[nb][j] = ColTile<CFG::RBB, ES>::lds_offset(krow, n / CE) + (n % CE) * ES;
-      }
-  }
-
-  // Read the fragments of k-slice kk of ring slot `slot`.
-  auto load_frags_b = [&](Frags<CFG>& f, int slot_off, int kk) {  // slot_off: byte offset of the ring slot
-    const char* sb = smem + slot_off + CFG::A_BYTES;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      if constexpr (CFG::B_KCONTIG) {
-#pragma unroll
-        for (int h = 0; h < NFRAG; ++h)
-          f.b[nb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sb + fb_off[kk][h] + nb * 32 * CFG::RBB);
-      } else if constexpr (CFG::IN == IN_FP8) {
-        i32x2_t t[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          t[r] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-              (LDS_AS i32x2_t*)(LDS_AS char*)(sb + fb_off[nb][0] + (kk * 64 + 8 * r) * CFG::RBB));
-        f.b[nb][0] = (i32x4_t){t[0].x, t[0].y, t[1].x, t[1].y};
-        f.b[nb][NFRAG - 1] = (i32x4_t){t[2].x, t[2].y, t[3].x, t[3].y};
-      } else {
-        i16x4_t t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (LDS_AS i16x4_t*)(LDS_AS char*)(sb + fb_off[nb][0] + kk * 16 * CFG::RBB));
-        i16x4_t t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (LDS_AS i16x4_t*)(LDS_AS char*)(sb + fb_off[nb][NTR - 1] + kk * 16 * CFG::RBB));
-        i32x2_t u0 = __builtin_bit_cast(i32x2_t, t0), u1 = __builtin_bit_cast(i32x2_t, t1);
-        f.b[nb][0] = (i32x4_t){u0.x, u0.y, u1.x, u1.y};
-      }
-    }
-  };
-  auto load_frags_a = [&](Frags<CFG>& f, int slot_off, int kk, int mb) {
-    const char* sa = smem + slot_off;
-#pragma unroll
-    for (int h = 0; h < NFRAG; ++h)
-      f.a[mb][h] = *(const LDS_AS i32x4_t*)(LDS_AS char*)(sa + fa_off[kk][h] + mb * 32 * CFG::RBA);
-  };
-  auto load_frags = [&](Frags<CFG>& f, int slot_off, int kk) {
-    load_frags_b(f, slot_off, kk);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) load_frags_a(f, slot_off, kk, mb);
-  };
-
-  const int total_tiles = p.tiles_m * p.tiles_n;
-  const int nsrc = (p.gather == GATHER_K) ? p.world : 1;
-  const int klocal = (p.gather == GATHER_K) ? p.K_local : p.K;
-  const int nkb = cdiv(klocal, BK);
-  const int nsteps = nsrc * nkb;
-  const unsigned smem_base = __builtin_amdgcn_readfirstlane(lds_address(smem));
-  const unsigned long long a_own = (unsigned long long)p.A;
-
-  for (int it = 0; ONE_ROUND ? it < 1 : true; ++it) {
-    const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
-    if (tidx < 0) break;
-    int tm, tn;
-    grouped_tile(tidx, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN;
-
-    // ---- per-tile loader state ---------------------------------------------------------------
-    // Row validity is folded into the per-lane offsets once per tile.
-    unsigned a_voff[LA], b_voff[LB];
-#pragma unroll
-    for (int i = 0; i < LA; ++i) a_voff[i] = (m0 + la_row[i] < p.M) ? la_off[i] : kInvalidOffset;
-#pragma unroll
-    for (int i = 0; i < LB; ++i) {
-      if constexpr (CFG::B_KCONTIG)
-        b_voff[i] = (n0 + lb_row[i] < p.N) ? lb_off[i] : kInvalidOffset;
-      else
-        b_voff[i] = (n0 + lb_col[i] < p.N) ? lb_off[i] : kInvalidOffset;
-    }
-    // Byte offset of this tile's first A row inside the slot that holds it.
-    int a_slot = p.rank;
-    long long a_row0 = m0;
-    if (p.gather == GATHER_M) {
-      a_slot = m0 / p.M_local;
-      a_row0 = m0 - (long long)a_slot * p.M_local;
-    }
-    if (p.gather == GATHER_K) a_slot = 0;
-    const unsigned long long a_tile_off = (unsigned long long)(a_row0 * p.s_am * ES);
-    const i32x4_t rb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)n0 * (CFG::B_KCONTIG ? p.s_bn : 1) * ES);
-    i32x4_t ra = make_rsrc_words((p.gather == GATHER_NONE ? a_own : in_slot(a_own, a_slot)) + a_tile_off);
-
-    // Loader position: next K step to issue = (i_src, i_kb), i_step overall.
-    int i_step = 0, i_src = 0, i_kb = 0;
-
-    // The direct-to-LDS loads of one K step, issued one at a time so that the main loop can spread
-    // them between its MFMAs (a wave issues in order: a burst of loads right after the barrier would
-    // hold back the MFMAs behind it while the memory pipeline absorbs the burst).  Steps past the end
-    // load nothing (every lane is out of range and deposits zeros), which keeps the per-thread count
-    // of outstanding loads identical on every step.
-    struct StepLoads {
-      int klim;
-      unsigned sa, sb, a_soff, b_soff;
-    };
-    auto begin_step = [&](int slot_off) {  // slot_off: byte offset of the ring slot to fill
-      StepLoads L;
-      const bool live = i_step < nsteps;
-      const int k0 = i_kb * BK;
-      L.klim = live ? klocal - k0 : 0;  // k elements of this step that exist
-      L.sa = smem_base + slot_off + wave * kDmaBytes;
-      L.sb = L.sa + CFG::A_BYTES;
-      L.a_soff = (unsigned)(k0 * ES);
-      const long long kglob = (long long)i_src * klocal + k0;
-      L.b_soff = __builtin_amdgcn_readfirstlane(
-          CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
-      return L;
-    };
-    auto load_offset = [&](const StepLoads& L, int j) -> unsigned {  // per-lane offset of load j
-      if (j < LA) return (la_k[j] < L.klim) ? a_voff[j] : kInvalidOffset;
-      const int i = j - LA;
-      const int kpos = CFG::B_KCONTIG ? lb_col[i] : lb_row[i];
-      return (kpos < L.klim) ? b_voff[i] : kInvalidOffset;
-    };
-    auto issue_at = [&](const StepLoads& L, int j, unsigned v) {
-      if (j < LA)
-        dma16(ra, L.sa + j * NW * kDmaBytes, v, L.a_soff);
-      else
-        dma16(rb, L.sb + (j - LA) * NW * kDmaBytes, v, L.b_soff);
-    };
-    auto issue_one = [&](const StepLoads& L, int j) { issue_at(L, j, load_offset(L, j)); };  // j in [0, LA + LB)
-    auto end_step = [&]() {
-      ++i_step;
-      if (++i_kb == nkb) {  // next source slot (gather along K only)
-        i_kb = 0;
-        ++i_src;
-        if (p.gather == GATHER_K && i_src < nsrc) ra = make_rsrc_words(in_slot(a_own, i_src) + a_tile_off);
-      }
-    };
-    auto issue = [&](int slot) {
-      const StepLoads L = begin_step(slot * CFG::STAGE_BYTES);
-#pragma unroll
-      for (int j = 0; j < LA + LB; ++j) issue_one(L, j);
-      end_step();
-    };
-
-    MfmaAcc<CFG> acc;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc.v[mb][nb][i] = 0.f;
-
-    // ---- prologue: fill STAGES-1 ring slots, wait for the first ----------------------------------
-    // The two-group loop reads a slot in both of its phases and refills it one step later than the
-    // single-group loop, so it keeps one step less in flight.
-    constexpr int AHEAD = PINGPONG ? STAGES - 2 : STAGES - 1;  // K steps issued before the loop starts
-#pragma unroll
-    for (int s = 0; s < AHEAD; ++s) issue(s);
-    wait_vmcnt<(AHEAD - 1) * (LA + LB)>();
-    __builtin_amdgcn_s_barrier();
-    Frags<CFG> fr[KS < 2 ? 2 : KS];  // one set per k-slice (two for the loops that double-buffer)
-    if constexpr (!PINGPONG) load_frags(fr[0], 0, 0);
-
-    // ---- main loop ----------------------------------------------------------------------------
-    // Invariant at the top of step s: the operands of step s are in LDS and visible to all waves,
-    // and the fragments of its first k-slice are in flight.  The step first makes sure step s+1
-    // has landed too, so that its first fragments can be fetched while step s still computes.
-    // The four-wave tiles have registers to spare and run the loop unrolled over the ring positions,
-    // which turns every LDS address of a step into a constant offset (5-10 % on those tiles); the
-    // eight-wave tile would spill and keeps the ring position in a register.
-    constexpr int RING_UNROLL = (NW == 4) ? STAGES : 1;
-    int s = 0, ring_pos = 0;
-    if constexpr (PINGPONG) {
-      // Eight waves, two per SIMD: waves 0-3 and waves 4-7 run half a step apart.  A step is a
-      // memory phase (all fragment reads of the step, then the direct-to-LDS loads that refill the
-      // slot of the previous step) and a compute phase (nothing but MFMAs), each closed by a
-      // workgroup barrier, so that on every SIMD one wave feeds the matrix pipe while the other
-      // one has the LDS and memory ports to itself.
-      const bool late = wave >= 4;
-      if (late) __builtin_amdgcn_s_barrier();
-      // The loader position of the common case - a whole K step inside one source - is carried in
-      // scalar registers that advance by constants, and its loads need no per-lane k test; partial
-      // steps, source changes and the empty steps past the end take the general path.
-      const unsigned b_inc = __builtin_amdgcn_readfirstlane(
-          CFG::B_KCONTIG ? (unsigned)(BK * ES) : (unsigned)((long long)BK * p.s_bk * ES));
-      unsigned a_so = 0, b_so = 0;
-      int k_left = 0;
-      auto resync = [&]() {
-        a_so = (unsigned)(i_kb * BK * ES);
-        const long long kglob = (long long)i_src * klocal + (long long)i_kb * BK;
-        b_so = __builtin_amdgcn_readfirstlane(
-            CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
-        k_left = i_step < nsteps ? klocal - i_kb * BK : 0;
-      };
-      resync();
-      unsigned rd = 0;                                    // byte offset of the slot this step reads
-      unsigned wr = AHEAD * CFG::STAGE_BYTES;             // ... and of the slot it refills
-      const unsigned wr_wave = smem_base + wave * kDmaBytes;
-      // The fragments of the first half of a step's MFMAs are read in the memory phase, those of the
-      // second half between the MFMAs of the first (LDS reads issue in the shadow of an MFMA;
-      // direct-to-LDS loads do not, a wave takes some 80 cycles to get one accepted).
-      constexpr int NMFMA = KS * MB * NB;
-      constexpr bool SPLIT_K = KS >= 2;                    // halves split by k-slice, else by row block
-      static_assert(KS == 1 || KS % 2 == 0, "k-slices split in two halves");
-      static_assert(MB % 2 == 0, "row blocks split in two halves");
-      // Late fragment reads, in pieces: per late k-slice the B fragments, then one row block of A each;
-      // with a single slice the upper row blocks of A.
-      constexpr int LATE_PIECES = SPLIT_K ? (KS / 2) * (1 + MB) : MB / 2;
-      auto late_piece = [&](int pc) {
-        if constexpr (SPLIT_K) {
-          const int kk = KS / 2 + pc / (1 + MB), q = pc % (1 + MB);
-          if (q == 0)
-            load_frags_b(fr[kk], rd, kk);
-          else
-            load_frags_a(fr[kk], rd, kk, q - 1);
-        } else {
-          load_frags_a(fr[0], rd, 0, MB / 2 + pc);
-        }
-      };
-      for (; s < nsteps; ++s) {
-        if constexpr (SPLIT_K) {
-#pragma unroll
-          for (int kk = 0; kk < KS / 2; ++kk) load_frags(fr[kk], rd, kk);
-        } else {
-          load_frags_b(fr[0], rd, 0);
-#pragma unroll
-          for (int mb = 0; mb < MB / 2; ++mb) load_frags_a(fr[0], rd, 0, mb);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (k_left >= BK) {
-#pragma unroll
-          for (int j = 0; j < LA; ++j) dma16(ra, wr_wave + wr + j * NW * kDmaBytes, a_voff[j], a_so);
-#pragma unroll
-          for (int i = 0; i < LB; ++i)
-            dma16(rb, wr_wave + wr + CFG::A_BYTES + i * NW * kDmaBytes, b_voff[i], b_so);
-        } else {
-          const StepLoads L = begin_step(wr);
-#pragma unroll
-          for (int j = 0; j < LA + LB; ++j) issue_one(L, j);
-        }
-        end_step();
-        if (i_kb == 0) {
-          resync();
-        } else {
-          a_so += BK * ES;
-          b_so += b_inc;
-          k_left -= BK;
-        }
-        // Own early fragment reads done and own loads of step s+1 landed.
-        wait_vmcnt_lgkm0<(AHEAD - 1) * (LA + LB)>();
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        // First half of the MFMAs with the late fragment reads spread between them.
-#pragma unroll
-        for (int i = 0; i < NMFMA / 2; ++i) {
-          const int kk = i / (MB * NB), mb = (i / NB) % MB, nb = i % NB;  // one slice: mb < MB/2 here
-          acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
-#pragma unroll
-          for (int pc = 0; pc < LATE_PIECES; ++pc)
-            if (pc * (NMFMA / 2) / LATE_PIECES == i) late_piece(pc);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int i = NMFMA / 2; i < NMFMA; ++i) {
-          const int kk = i / (MB * NB), mb = (i / NB) % MB, nb = i % NB;
-          acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(fr[kk].a[mb], fr[kk].b[nb], acc.v[mb][nb]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        rd = rd + CFG::STAGE_BYTES == CFG::RING_BYTES ? 0 : rd + CFG::STAGE_BYTES;
-        wr = wr + CFG::STAGE_BYTES == CFG::RING_BYTES ? 0 : wr + CFG::STAGE_BYTES;
-      }
-      if (!late) __builtin_amdgcn_s_barrier();
-    } else
-    while (s < nsteps) {
-#pragma unroll
-    for (int u = 0; u < RING_UNROLL; ++u) {
-      if (s >= nsteps) break;
-      ++s;
-      const int slot = (RING_UNROLL == 1) ? ring_pos : u;
-      // LDS is one coherent memory per CU, so a bare s_barrier (no fence, hence no forced wait for
-      // the fragment reads in flight) orders the operand ring between the waves.
-      wait_vmcnt<(STAGES - 3) * (LA + LB)>();  // this thread's loads of step s+1 have landed
-      __builtin_amdgcn_s_barrier();             // everyone's have; everyone is past step s-1
-      int pslot = slot + STAGES - 1;
-      if (pslot >= STAGES) pslot -= STAGES;
-      const StepLoads L = begin_step(pslot * CFG::STAGE_BYTES);  // refills the slot the previous step used
-      const int nslot = slot + 1 == STAGES ? 0 : slot + 1;
-      constexpr int NSLOT = KS * MB;          // MFMA groups of a step; the loads are spread over them
-      constexpr int NLOAD = LA + LB;
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) {
-        if (kk + 1 < KS)
-          load_frags(fr[(kk + 1) & 1], slot * CFG::STAGE_BYTES, kk + 1);
-        else
-          load_frags(fr[(kk + 1) & 1], nslot * CFG::STAGE_BYTES, 0);
-        const Frags<CFG>& f = fr[kk & 1];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-          for (int j = 0; j < NLOAD; ++j)
-            if (j * NSLOT / NLOAD == kk * MB + mb) issue_one(L, j);
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) acc.v[mb][nb] = mfma_block<CFG::IN, NFRAG>(f.a[mb], f.b[nb], acc.v[mb][nb]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      end_step();
-      static_assert(KS % 2 == 0 || KS == 1, "fragment double buffer assumes an even slice count");
-      if constexpr (KS == 1) {
-        // With one slice per step the two buffers alternate across steps.
-        Frags<CFG> t = fr[0];
-        fr[0] = fr[1];
-        fr[1] = t;
-      }
-      ring_pos = nslot;
-    }
-    }
-
-    // The ring is reused as epilogue staging: drain the (empty) loads still in flight and make
-    // sure every wave has finished reading operands.
-    wait_vmcnt<0>();
-    __syncthreads();
-
-    // ---- epilogue -------------------------------------------------------------------------------
-    // The whole output tile is first written to LDS in the output type (the operand ring is dead
-    // by now), which frees the accumulators; both phases then stream rows of the tile, 16 bytes per
-    // lane and BN*2 contiguous bytes per row, with many loads in flight per thread.
-    {
-      float badd[MB];
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        badd[mb] = 0.f;
-        if (p.bias) {
-          const int gm = m0 + wm * TM + mb * 32 + acc_col(lane);
-          if (gm < p.M) badd[mb] = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
-        }
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            unsigned short h[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              h[e] = Out::from_float(acc_read(acc.v[mb][nb][4 * q + e]) * p.scale + badd[mb]);
-            u32x2_t w;
-            w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
-            w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
-            const int trow = wm * TM + mb * 32 + acc_col(lane);
-            const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
-            *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
-          }
-    }
-    __syncthreads();
-
-    constexpr int CPR = BN / 8;            // 16-byte chunks per tile row
-    constexpr int RPP = NT / CPR;          // tile rows covered by one pass of the workgroup
-    constexpr int PASSES = BM / RPP;
-    const int t_row = tid / CPR, t_chunk = tid % CPR;
-    const int gn = n0 + t_chunk * 8;
-    const bool col_ok = gn < p.N;
-    const char* const t_lds = smem + t_row * CFG::TROW + t_chunk * 16;
-
-    // Phase 1: C (plain store) or aux (own slot).  When no peer contributes (world of one, or peers
-    // switched off) the reduced tile equals the own tile, so C is written in the same pass and
-    // phase 2 is skipped.
-    const bool flags = epi_has_flags(p.epi);
-    const bool solo = flags && (!p.sum_peers || p.world == 1);
-    {
-      char* const out1 = flags ? p.aux : p.C;
-      const int ftn1 = cdiv(p.N, p.flag_bn);
-      const int ftotal1 = cdiv(p.M, p.flag_bm) * ftn1;
-      const unsigned long long c_base = (unsigned long long)p.C;
-#pragma unroll 4
-      for (int ps = 0; ps < PASSES; ++ps) {
-        const int gm = m0 + ps * RPP + t_row;
-        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + ps * RPP * CFG::TROW);
-        if (gm < p.M && col_ok) {
-          const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gn) * 2;
-          if (p.epi == EPI_ALL_GATHER) {
-            // the tile goes to every rank's gathered output (iris/mem/triton/context.py:841-864)
-            for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
-          } else if (p.epi == EPI_ATOMIC) {
-            // the tile is added into every rank's C (iris/mem/triton/context.py:689-702)
-            for (int pr = 0; pr < p.world; ++pr) {
-              char* dst = (char*)(in_slot(c_base, pr) + eoff);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) atomic_add_packed<Out>(dst + 4 * e, v[e]);
-            }
-          } else if (flags) {
-            store16_system(out1 + eoff, v);  // aux: read by the peers as soon as the flag is up
-          } else {
-            *(u32x4_t*)(out1 + eoff) = v;
-          }
-          if (solo) {
-            int owner = p.rank;
-            if (p.epi != EPI_ONE_SHOT) owner = owner_of(p.epi, (gm / p.flag_bm) * ftn1 + gn / p.flag_bn, ftotal1, p.world, p.rank);
-            if (p.all_owners || owner == p.rank) {
-              if (p.epi == EPI_TWO_SHOT) {
-                for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
-              } else {
-                const int dst = p.all_owners ? owner : p.rank;
-                *(u32x4_t*)(in_slot(c_base, dst) + eoff) = v;
-              }
-            }
-          }
-        }
-      }
-    }
-
-    if (flags) {
-      // Publish: the aux tile was stored write-through at system scope; every wave waits until its
-      // stores are acknowledged, the workgroup meets, and the threads that own flags raise them
-      // (no L2 write-back is needed any more).  Likewise the peers' flags are polled (system-scope
-      // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
-      // every wave poll and run ahead measured slower.
-      wait_vmcnt<0>();
-      __syncthreads();
-      raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
-      if (!solo) {
-        wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
-        __syncthreads();
-      }
-
-      // Phase 2: reduce the flag tiles this rank is responsible for.  The peer loads are issued
-      // unconditionally (rows this thread does not reduce read the tile origin instead) and for a
-      // compile-time number of peers, so that all loads of a group of passes are in flight
-      // together; only the stores are predicated.
-      const bool ref_chain = (p.acc_mode == IRIS_HIP_ACC_REFERENCE) && !Out::kFp32SumInReference;
-      const unsigned long long aux_own = (unsigned long long)p.aux, c_own = (unsigned long long)p.C;
-      const int ftn = cdiv(p.N, p.flag_bn);
-      const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
-      const int fcol = gn / p.flag_bn;
-      const int npeers = p.sum_peers ? p.world - 1 : 0;
-      // Peer aux bases in ascending rank order, own rank skipped.
-      unsigned long long pb[kMaxCachedSlots - 1];
-#pragma unroll
-      for (int i = 0; i < kMaxCachedSlots - 1; ++i) pb[i] = (i < p.rank ? hb[i] : hb[i + 1]) + (aux_own - hb_own);
-      const long long safe_off = ((long long)m0 * p.s_cm + n0) * 2;  // first element of the tile
-
-      auto reduce_tile = [&](auto np_tag, auto nt_tag) {
-        constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
-        constexpr bool NT = decltype(nt_tag)::value;  // peers' tiles and C bypass the caches' keep policy
-        constexpr int NPV = NP > 0 ? NP : 1;
-        // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
-        // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
-        // at a time also with seven peers, and groups below the last row of the matrix are skipped.
-        constexpr int G = (NP >= 4 && NW == 8) ? 2 : 4;
-        static_assert(PASSES % G == 0, "pass grouping");
-        for (int pg = 0; pg < PASSES; pg += G) {
-          if (m0 + pg * RPP >= p.M) break;
-          bool active[G];
-          long long eoff[G];
-          int owner[G];
-          u32x4_t own[G], pv[G][NPV];
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const int gm = m0 + (pg + g) * RPP + t_row;
-            owner[g] = p.rank;
-            if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
-              const int t = (gm / p.flag_bm) * ftn + fcol;
-              owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
-            }
-            active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
-            eoff[g] = active[g] ? ((long long)gm * p.s_cm + gn) * 2 : safe_off;
-            if constexpr (NP > 0) {
-#pragma unroll
-              for (int i = 0; i < NP; ++i) {
-                if constexpr (NT) pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
-                else pv[g][i] = *(const u32x4_t*)(pb[i] + eoff[g]);
-              }
-            }
-            own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
-          }
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            float sum[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              sum[2 * e] = Out::to_float((unsigned short)(own[g][e] & 0xFFFF));
-              sum[2 * e + 1] = Out::to_float((unsigned short)(own[g][e] >> 16));
-            }
-            auto add_peer = [&](const u32x4_t& v) {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
-                sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
-              }
-              if (ref_chain) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
-              }
-            };
-            if constexpr (NP > 0) {
-#pragma unroll
-              for (int i = 0; i < NP; ++i) add_peer(pv[g][i]);
-            } else if constexpr (NP < 0) {
-              for (int pr = 0; pr < p.world; ++pr)
-                if (pr != p.rank) add_peer(*(const u32x4_t*)(in_slot(aux_own, pr) + eoff[g]));
-            }
-            u32x4_t res;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
-            if (active[g]) {
-              if (p.epi == EPI_TWO_SHOT) {
-                *(u32x4_t*)(c_own + eoff[g]) = res;
-                for (int pr = 0; pr < p.world; ++pr)
-                  if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
-              } else {
-                const int dst = p.all_owners ? owner[g] : p.rank;
-                u32x4_t* cdst = (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]);
-                if constexpr (NT) __builtin_nontemporal_store(res, cdst);
-                else *cdst = res;
-              }
-            }
-          }
-        }
-      };
-      switch (solo ? -2 : (p.world <= kMaxCachedSlots ? npeers : -1)) {
-        case -2: break;  // C was written in phase 1
-        case 1: reduce_tile(std::integral_constant<int, 1>{}, std::false_type{}); break;
-        case 3: reduce_tile(std::integral_constant<int, 3>{}, std::false_type{}); break;
-        case 7:
-          // Peer tiles are read once; when they exceed what the last-level cache holds, streaming
-          // them non-temporally is faster (measured: 663 -> 622 us for 7 x 256 MiB of peers), for
-          // smaller launches it is not (two-shot 4096 x 4096: 91 -> 98 us).
-          if (p.stream_peers) reduce_tile(std::integral_constant<int, 7>{}, std::true_type{});
-          else reduce_tile(std::integral_constant<int, 7>{}, std::false_type{});
-          break;
-        default: reduce_tile(std::integral_constant<int, -1>{}, std::false_type{}); break;
-      }
-    }
-    // Staging shares LDS with the operand ring of the next tile: every wave must be done reading it.
-    // A bare barrier - __syncthreads() would also wait for this tile's global stores to be
-    // acknowledged (1-4 us), which nothing here depends on; they drain behind the next tile's
-    // first loads, or behind the end of the kernel.
-    __builtin_amdgcn_s_waitcnt((0xF) | (0x3 << 14) | (0x7 << 4));  // lgkmcnt(0), vmcnt and expcnt free
-    __builtin_amdgcn_s_barrier();
-  }
-}
+#include "fused_kernel.h"
 
 // ------------------------------------------------------------------------------------------------
 // Generic kernel: 64x64 tile, 256 threads, 4x4 outputs per thread, fp32 FMA.
@@ -1183,40 +279,6 @@ const char* mfma_ineligible(const FusedParams& p, int in_dtype, int out_dtype, i
   return nullptr;
 }
 
-template <class CFG, bool ONE_ROUND>
-int launch_mfma_grid(const FusedParams& p, int device, int grid, hipStream_t stream) {
-  // The dynamic-LDS limit is a per-device attribute of the kernel: set it once on every device used.
-  static bool attr_set[64] = {};
-  if (!attr_set[device]) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG, ONE_ROUND>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_set[device] = true;
-  }
-  hipLaunchKernelGGL((fused_mfma_kernel<CFG, ONE_ROUND>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
-  return (int)hipGetLastError();
-}
-
-template <class CFG>
-int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stream, const char* name) {
-  const int total = p.tiles_m * p.tiles_n;
-  const int cap = cu_count * CFG::WG_PER_CU;
-  // A multiple of the XCD count keeps the XCD mapping exact.  Rounded up when the tiles fit in one
-  // round (the surplus workgroups find no tile and leave), so that no tile waits for a second round.
-  int grid = total < cap ? total : cap;
-  if (grid % p.num_xcd) {
-    const int up = grid + p.num_xcd - grid % p.num_xcd;
-    grid = up <= cap ? up : grid - grid % p.num_xcd;
-  }
-  if (grid < 1) grid = 1;
-  snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name);
-  // The one-round build exists for the latency-bound tiles only (one workgroup of four waves per CU).
-  if constexpr (CFG::NW == 4 && CFG::WG_PER_CU == 1) {
-    if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
-  }
-  return launch_mfma_grid<CFG, false>(p, device, grid, stream);
-}
-
 template <class In, class Out>
 int launch_generic(FusedParams p, int cu_count, hipStream_t stream, const char* name) {
   p.tiles_m = cdiv(p.M, GT);
@@ -1242,57 +304,14 @@ int dispatch_generic(const FusedParams& p, int in_dtype, int out_dtype, int cu, 
   return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
 }
 
-// Tile shapes of the MFMA kernel.
-//   big     256x256, 8 waves, 4-slot ring: 128 accumulator registers per lane, the shape for large
-//           problems (half the operand bytes per flop of the 128x128 tiles).
-//   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
-//   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
-// Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
-// smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
-//   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
-//           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
-//           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
-//           tiles the shorter K steps make it the slower of the two.
-enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3 };
-constexpr int tile_bk(int kind, int in) {  // K elements per step
-  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
-}
-template <int IN, bool BKC>
-using BigTile = MfmaCfg<IN, 256, 256, tile_bk(TILE_BIG, IN), 2, 4, 4, BKC>;
-template <int IN, bool BKC>
-using SmallTile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL, IN), 2, 2, 4, BKC>;
-template <int IN, bool BKC>
-using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
-template <int IN, bool BKC>
-using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
+}  // namespace
 
-inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SKINNY ? 64 : 128; }
-inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : 128; }
+// Instantiated in iris_hip_mfma_bf16.hip, iris_hip_mfma_f16.hip and iris_hip_mfma_fp8.hip.
+extern template int dispatch_mfma_in<IN_BF16>(FusedParams&, int, bool, int, int, hipStream_t);
+extern template int dispatch_mfma_in<IN_F16>(FusedParams&, int, bool, int, int, hipStream_t);
+extern template int dispatch_mfma_in<IN_FP8>(FusedParams&, int, bool, int, int, hipStream_t);
 
-template <int IN>
-int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hipStream_t s) {
-  const int bm = tile_rows(kind), bn = tile_cols(kind);
-  p.tiles_m = cdiv(p.M, bm);
-  p.tiles_n = cdiv(p.N, bn);
-  // Group height: tile-rows walked together so that an XCD's span of tiles is close to square.
-  const int span = cdiv(p.tiles_m * p.tiles_n, p.num_xcd);
-  int g = 1;
-  while (g * g * 2 <= span && g * 2 <= p.tiles_m) g *= 2;
-  p.group_m = g;
-  static const char* names[3] = {"bf16", "f16", "fp8"};
-  char name[96];
-  snprintf(name, sizeof(name), "mfma_%s_%dx%dx%d_%s", names[IN], bm, bn, tile_bk(kind, IN), bkc ? "nt" : "nn");
-  switch (kind) {
-    case TILE_BIG:
-      return bkc ? launch_mfma<BigTile<IN, true>>(p, device, cu, s, name) : launch_mfma<BigTile<IN, false>>(p, device, cu, s, name);
-    case TILE_SMALL:
-      return bkc ? launch_mfma<SmallTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, device, cu, s, name);
-    case TILE_SMALL2:
-      return bkc ? launch_mfma<Small2Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, device, cu, s, name);
-    default:
-      return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, device, cu, s, name);
-  }
-}
+namespace {
 
 int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
   g_last_error[0] = 0;
