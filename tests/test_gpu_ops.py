@@ -550,6 +550,42 @@ def test_tile_counts_off_the_xcd_multiple(M, N, K, tile):
         assert_bits_equal(got[r], exp["C"][r], f"{kernel} C in slot {r}")
 
 
+# Seeded random draws over world size, rank, element type, shape (all four tile shapes), variant and
+# flag-tile size; integer-valued operands, so every output bit is determined.
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_bit_exact(seed):
+    import random
+
+    rng = random.Random(seed)
+    for case in range(10):
+        W = rng.choice([1, 2, 3, 4, 8])
+        rank = rng.randrange(W)
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        if rng.random() < 0.3:
+            M, N, K = rng.choice([2304, 2560, 4100]), rng.choice([3584, 4096, 2312]), rng.choice([8, 40, 136])
+        else:
+            M = rng.choice([1, 17, 32, 33, 64, 96, 130, 200, 384, 640, 1000])
+            N = rng.choice([64, 72, 136, 264, 520, 1152, 2880])
+            K = rng.choice([8, 24, 72, 128, 200, 520])
+        variant = rng.choice(["one_shot", "two_shot"])
+        bm = min(rng.choice([16, 32, 64, 128]), M) if M >= 16 else 1
+        bn = min(rng.choice([32, 64, 128]), N)
+        what = f"seed {seed} case {case}: W={W} rank={rank} {dtype} {M}x{N}x{K} {variant} flags {bm}x{bn}"
+        ctx = _ctx(W, rank, heap=1 << 27)
+        A, B = randint_cpu((M, K), 1000 + case, dtype), randint_cpu((K, N), 2000 + case, dtype)
+        peers = [randn_cpu((M, N), 3000 + 10 * case + r, dtype) for r in range(W)]
+        cfg = iris.FusedConfig(block_size_m=bm, block_size_n=bn, block_size_k=8, all_reduce_variant=variant)
+        dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg)
+        assert kernel.startswith("mfma_"), f"{what}: {kernel}"
+        exp = oracle.matmul_all_reduce(A, B, peers, rank, W, bm, bn, variant, "fp32")
+        assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"{what}: aux")
+        assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), f"{what}: flags"
+        for r, got in enumerate(slot_copies(ctx, dC)):
+            assert_bits_equal(got, exp["C"][r], f"{what}: {kernel} C in slot {r}")
+        del ctx, dC, ws
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("M,N,K", [(200, 272, 80), (1, 1024, 256), (520, 144, 1008)])
 def test_ragged_shapes_mfma_fp8(M, N, K):
     W, rank = 4, 1
