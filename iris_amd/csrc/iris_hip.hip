@@ -203,13 +203,7 @@ namespace {
 thread_local char g_last_error[512] = "";
 thread_local char g_last_kernel[128] = "";
 
-int fail(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
-  va_end(ap);
-  return (int)hipErrorInvalidValue;
-}
+using iris_host::fail;  // defined below, shared with the other translation units
 
 struct DeviceFacts {
   int cu_count = 0;
