@@ -949,8 +949,8 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   }
   if (grid < 1) grid = 1;
   iris_host::set_last_kernel(name);
-  // The one-round build exists for the latency-bound tiles only (one workgroup of four waves per CU).
-  if constexpr (CFG::NW == 4 && CFG::WG_PER_CU == 1) {
+  // The one-round build exists for the tiles that run one workgroup per CU.
+  if constexpr (CFG::WG_PER_CU == 1) {
     if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
   }
   return launch_mfma_grid<CFG, false>(p, device, grid, stream);
