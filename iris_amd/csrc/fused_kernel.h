@@ -949,10 +949,7 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   }
   if (grid < 1) grid = 1;
   iris_host::set_last_kernel(name);
-  // The one-round build exists for the tiles that run one workgroup per CU.
-  if constexpr (CFG::WG_PER_CU == 1) {
-    if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
-  }
+  if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
   return launch_mfma_grid<CFG, false>(p, device, grid, stream);
 }
 
