@@ -950,6 +950,16 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   if (grid < 1) grid = 1;
   iris_host::set_last_kernel(name);
   if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
+  // More tiles than workgroups that fit at once: normally the resident workgroups loop over the tiles.
+  // The two-shot all-reduce does better with one workgroup per tile, handed out by the hardware as CUs
+  // free up (measured at W = 8: 16384x4096x1376 322 -> 273 us, 8192x8192x2752 461 -> 417 us,
+  // 8192x8192x8192 1059 -> 1009 us); the one-shot variant does worse that way (+3-7 %), launches
+  // without peers do not care.
+  if (p.epi == EPI_TWO_SHOT && p.world > 1 && p.sum_peers) {
+    int per_tile = total;
+    if (per_tile % p.num_xcd) per_tile += p.num_xcd - per_tile % p.num_xcd;
+    return launch_mfma_grid<CFG, true>(p, device, per_tile, stream);
+  }
   return launch_mfma_grid<CFG, false>(p, device, grid, stream);
 }
 
