@@ -37,8 +37,10 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
                                                  (tests/ccl/test_all_reduce.py:55,92-97), equality with a
                                                  plain fp32 sum for exactly representable data, and the
                                                  one-shot order against a sequential Python sum.  The
-                                                 rotated start rank of two-shot is source-pinned only (no
-                                                 reference test can see it): parity unpinned by tests
+                                                 rotated start rank of two-shot is pinned by a literal
+                                                 replay of the reference's program loop (pid over
+                                                 COMM_SMS, start = pid % W) on order-sensitive fp32 data
+                                                 and by hand-worked known answers per start rank
   quantize_e4m3 / fp8 products                  no reference counterpart (the reference has no fp8
                                                  path): defined by the target configuration itself (e4m3fn inputs with
                                                  per-tensor scales amax/448, fp32 accumulation), parity unpinned

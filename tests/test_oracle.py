@@ -335,3 +335,92 @@ def test_ccl_two_shot_with_one_workgroup_starts_every_tile_at_rank_zero():
     for r in range(4):
         outs = oracle.ccl_all_reduce(inputs, outs, r, "two_shot", block_m=32, block_n=32, comm_sms=1, distribution=0)
     assert all(torch.all(o == 0.0) for o in outs)
+
+
+def _two_shot_program_replay(inputs, group_rank, block_m, block_n, group_m, comm_sms, distribution):
+    """The reference kernel's loop written out program by program
+    (iris/ccl/triton/all_reduce.py:602-669): programs pid = 0..COMM_SMS-1, each walking
+    range(pid, max_tile_offset, COMM_SMS), every tile summed from start = pid % W going round the
+    ranks, element by element in numpy float32.  Shares no code with oracle.ccl_*."""
+    W = len(inputs)
+    M, N = inputs[0].shape
+    x = [t.to(torch.float32).numpy() for t in inputs]
+    num_pid_m, num_pid_n = -(-M // block_m), -(-N // block_n)
+    total_tiles = num_pid_m * num_pid_n
+    tiles_per_rank = -(-total_tiles // W)
+    if distribution == 0:
+        start_tile, stride = group_rank, W
+        max_tile_offset = -(-max(total_tiles - start_tile, 0) // stride)
+    else:
+        start_tile, stride = group_rank * tiles_per_rank, 1
+        max_tile_offset = min(tiles_per_rank, max(total_tiles - start_tile, 0))
+    out = np.full((M, N), np.nan, dtype=np.float32)
+    for pid in range(comm_sms):
+        for tile_offset in range(pid, max_tile_offset, comm_sms):
+            tile_id = start_tile + tile_offset * stride
+            num_pid_in_group = group_m * num_pid_n
+            group_id = tile_id // num_pid_in_group
+            first_pid_m = group_id * group_m
+            group_size_m = min(num_pid_m - first_pid_m, group_m)
+            pid_m = first_pid_m + ((tile_id % num_pid_in_group) % group_size_m)
+            pid_n = (tile_id % num_pid_in_group) // group_size_m
+            start_rank_idx = pid % W
+            for m in range(pid_m * block_m, min((pid_m + 1) * block_m, M)):
+                for n in range(pid_n * block_n, min((pid_n + 1) * block_n, N)):
+                    acc = np.float32(x[start_rank_idx][m, n])
+                    for i in range(1, W):
+                        acc = np.float32(acc + x[(start_rank_idx + i) % W][m, n])
+                    assert np.isnan(out[m, n]), "an element is reduced by one program only"
+                    out[m, n] = acc
+    return out
+
+
+def test_ccl_two_shot_rotation_known_answers():
+    # 2^24, -2^24, 0.5, 1 summed cyclically in fp32 gives a different value from every start rank:
+    #   start 0: (2^24 - 2^24) + 0.5 + 1               = 1.5
+    #   start 1: (-2^24 + 0.5 -> -2^24) + 1 -> -2^24+1 exactly; + 2^24 = 1
+    #   start 2: 0.5 + 1 = 1.5; + 2^24 -> 2^24 + 2 (nearest); - 2^24 = 2
+    #   start 3: 1 + 2^24 -> 2^24 (tie to even); - 2^24 = 0; + 0.5 = 0.5
+    vals = [2.0 ** 24, -(2.0 ** 24), 0.5, 1.0]
+    by_start = {0: 1.5, 1: 1.0, 2: 2.0, 3: 0.5}
+    W, bm, bn = 4, 2, 4
+    M, N = 2, 4 * 24  # one tile-row of 24 tiles, rank 0 owns tiles 0, 4, 8, ... (strided)
+    inputs = [torch.full((M, N), v, dtype=torch.float32) for v in vals]
+    outs = [torch.zeros((M, N)) for _ in vals]
+    for comm_sms in (3, 5):
+        got = oracle.ccl_all_reduce(inputs, outs, 0, "two_shot", block_m=bm, block_n=bn, group_m=1,
+                                    comm_sms=comm_sms, distribution=0)
+        # the j-th owned tile (tile id 4j) is handled by program j mod comm_sms
+        for j in range(6):
+            want = by_start[(j % comm_sms) % W]
+            for r in range(W):  # the owner stores the tile into every rank's output
+                assert torch.all(got[r][:, 16 * j:16 * j + 4] == want), (comm_sms, j, r)
+
+
+@pytest.mark.parametrize("distribution", [0, 1])
+@pytest.mark.parametrize("comm_sms", [3, 5])
+def test_ccl_two_shot_matches_the_program_loop(comm_sms, distribution):
+    W, M, N, bm, bn, gm = 4, 22, 40, 4, 8, 2  # ragged tiles, a short last group
+    g = torch.Generator().manual_seed(17)
+    # magnitudes spread over 2^0 .. 2^26 with both signs: almost every element's fp32 sum depends on the order
+    inputs = [(torch.randn((M, N), generator=g) * 2.0 ** torch.randint(0, 27, (M, N), generator=g).float())
+              for _ in range(W)]
+    covered = np.zeros((M, N), dtype=np.int32)
+    differs = 0
+    for rank in range(W):
+        want = _two_shot_program_replay(inputs, rank, bm, bn, gm, comm_sms, distribution)
+        own = ~np.isnan(want)
+        covered += own
+        before = torch.full((M, N), -7.0)
+        got = oracle.ccl_reduce_scatter(inputs, before, rank, bm, bn, gm, comm_sms, distribution).numpy()
+        assert np.array_equal(got[own].view(np.int32), want[own].view(np.int32))
+        assert np.all(got[~own] == -7.0)
+        outs = oracle.ccl_all_reduce(inputs, [before.clone() for _ in range(W)], rank, "two_shot", bm, bn, gm,
+                                     comm_sms, distribution)
+        for r in range(W):
+            assert np.array_equal(outs[r].numpy()[own].view(np.int32), want[own].view(np.int32))
+            assert np.all(outs[r].numpy()[~own] == -7.0)
+        ascending = sum(x.numpy().astype(np.float32) for x in inputs)  # fixed start at rank 0
+        differs += int(np.sum(ascending[own] != want[own]))
+    assert np.all(covered == 1)
+    assert differs > 50, "the data must tell the rotated order from the ascending one"
