@@ -10,6 +10,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "iris_hip.h"
@@ -924,13 +925,15 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 // ------------------------------------------------------------------------------------------------
 template <class CFG, bool ONE_ROUND>
 int launch_mfma_grid(const FusedParams& p, int device, int grid, hipStream_t stream) {
-  // The dynamic-LDS limit is a per-device attribute of the kernel: set it once on every device used.
-  static bool attr_set[64] = {};
-  if (!attr_set[device]) {
+  // The dynamic-LDS limit is a per-device attribute of the kernel: set it once on every device used
+  // (atomic flags: two host threads may both set it, which is harmless, but neither skips it).
+  static std::atomic<bool> attr_set[64];
+  if (device < 0 || device >= 64) return iris_host::fail("device index %d out of range", device);
+  if (!attr_set[device].load(std::memory_order_acquire)) {
     hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG, ONE_ROUND>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
     if (e != hipSuccess) return (int)e;
-    attr_set[device] = true;
+    attr_set[device].store(true, std::memory_order_release);
   }
   hipLaunchKernelGGL((fused_mfma_kernel<CFG, ONE_ROUND>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
   return (int)hipGetLastError();

@@ -30,6 +30,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "fused_kernel.h"
@@ -213,9 +214,11 @@ struct DeviceFacts {
 };
 
 DeviceFacts g_facts[64];
+std::mutex g_facts_mutex;  // entry points may be called from several host threads
 
 int facts_for(int device, DeviceFacts** out) {
   if (device < 0 || device >= 64) return fail("device index %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_facts_mutex);
   DeviceFacts& f = g_facts[device];
   if (!f.ok) {
     hipDeviceProp_t prop;
@@ -223,8 +226,14 @@ int facts_for(int device, DeviceFacts** out) {
     if (e != hipSuccess) return (int)e;
     f.cu_count = prop.multiProcessorCount;
     f.lds_per_block = (int)prop.sharedMemPerBlock;
-    // MI300/MI350-class parts expose 8 XCDs; smaller parts have one.
-    f.xcc_count = (f.cu_count >= 64 && f.cu_count % 8 == 0) ? 8 : 1;
+    // XCD count as the runtime reports it (the reference asks the same attribute,
+    // iris/host/platform/hip.py:218-231); a runtime that does not know the attribute means one XCD.
+    int xcc = 0;
+    if (hipDeviceGetAttribute(&xcc, hipDeviceAttributeNumberOfXccs, device) != hipSuccess || xcc < 1) {
+      (void)hipGetLastError();
+      xcc = 1;
+    }
+    f.xcc_count = xcc;
     f.ok = true;
   }
   *out = &f;
@@ -319,7 +328,8 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     p.flag_bm = 256;  // no flags on this path; any valid tile size
     p.flag_bn = 64;
   }
-  if ((p.world > 1 || p.gather != GATHER_NONE) && !p.heap_bases) return fail("context_tensor must not be NULL");
+  // Every kernel translates addresses through the heap bases, also with one rank.
+  if (!p.heap_bases) return fail("context_tensor must not be NULL");
   if (elem_size(in_dtype) == 0 || elem_size(out_dtype) == 0 || out_dtype == IRIS_HIP_FP8_E4M3)
     return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
 

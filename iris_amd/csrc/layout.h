@@ -15,7 +15,7 @@
 //   "col tile"   an operand tile stored as [BK rows (k)][BN elements], N contiguous (row-major B)
 #pragma once
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define IRIS_HD __host__ __device__ __forceinline__
 #else
 #define IRIS_HD inline

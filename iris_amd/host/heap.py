@@ -20,15 +20,30 @@ from .logging import log_rank
 
 class _DeviceSpan:
     """Expose raw device memory to torch through the CUDA array interface
-    (the reference's CUDAArrayInterface / tensor_from_ptr, iris/host/memory/tensor_utils.py:60-135)."""
+    (the reference's CUDAArrayInterface / tensor_from_ptr, iris/host/memory/tensor_utils.py:60-135).
 
-    def __init__(self, ptr, nbytes):
+    The span owns the allocation: torch keeps a reference to this object for as long as any tensor
+    made from it (or any view of one) is alive, so the memory is released when the last such tensor
+    goes away and never earlier - a tensor from ctx.zeros() may outlive its context, as it may in the
+    reference, whose torch allocator keeps the heap alive through the tensors' storage.
+    """
+
+    def __init__(self, ptr, nbytes, release=None):
+        self._ptr, self._release = ptr, release
         self.__cuda_array_interface__ = {
             "shape": (nbytes,),
             "typestr": "|u1",
             "data": (ptr, False),
             "version": 3,
         }
+
+    def __del__(self):
+        release, self._release = self._release, None
+        if release is not None and self._ptr:
+            try:
+                release(self._ptr)
+            except Exception:  # interpreter shutdown: the runtime may be gone already
+                pass
 
 
 class SymmetricHeap:
@@ -64,7 +79,7 @@ class SymmetricHeap:
             hip.set_device(device_id)
             self._raw_ptr = hip.hip_malloc(total)
             self.device = torch.device(f"cuda:{device_id}")
-            self._pool = torch.as_tensor(_DeviceSpan(self._raw_ptr, total), device=self.device)
+            self._pool = torch.as_tensor(_DeviceSpan(self._raw_ptr, total, hip.hip_free), device=self.device)
             base = self._raw_ptr
         elif backing == "host":
             self.device = torch.device("cpu")
@@ -145,13 +160,10 @@ class SymmetricHeap:
         return self._view(rank, offset, nbytes, tensor.dtype).reshape(tensor.shape)
 
     def close(self):
-        if self._raw_ptr:
-            ptr, self._raw_ptr = self._raw_ptr, 0
-            self._pool = None
-            try:
-                hip.hip_free(ptr)
-            except Exception:
-                pass
+        """Drop this object's references.  The device memory itself is released by the span object
+        that torch holds, once the last tensor on the heap is gone."""
+        self._raw_ptr = 0
+        self._pool = None
 
     def __del__(self):
         self.close()

@@ -1,9 +1,9 @@
 """The five target configurations of this build at full size on the GPU, against the CPU oracle.
 
 Inputs are drawn on the CPU from torch.Generator().manual_seed(seed) as the configurations state.
-Full-size comparisons use the oracle directly where it finishes in seconds; the largest case (fp8,
-16384 x 8192) is checked on row blocks plus size-independent properties (flags all raised, aux equal
-to the own product, untouched slots untouched).
+Full-size comparisons use the oracle directly; the largest case (fp8, 16384 x 8192) is compared in row
+chunks that cover the whole output, plus size-independent properties (flags all raised, untouched slots
+untouched).
 """
 
 import pytest
@@ -125,6 +125,42 @@ def test_config4_matmul_reduce_scatter_bf16():
         assert torch.all(got[r][other] == 0), f"slot {r} holds rows it does not own"
 
 
+@pytest.mark.parametrize("rank", [0, 7])
+def test_config4_matmul_reduce_scatter_accumulate_leg(rank):
+    """The reference semantics at full size (iris/mem/triton/context.py:953-997): one rank's launch,
+    seven staged peer aux buffers, the rank's 1024-row block summed over the slots in fp32 and cast once."""
+    M, N, K, W = 8192, 4096, 1376, 8
+    g = torch.Generator().manual_seed(0)
+    A = (torch.randn((M, K), generator=g) / K ** 0.5).to(torch.bfloat16)
+    B = (torch.randn((K, N), generator=g) / K ** 0.5).to(torch.bfloat16)
+    peers = [None if r == rank else randn_cpu((M, N), 1 + r, torch.bfloat16) for r in range(W)]
+    ctx = iris.iris(1 << 28, num_ranks=W, rank=rank)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=torch.bfloat16)
+    for r in range(W):
+        ctx.peer_view(dC, r).zero_()
+    ws = ops.matmul_reduce_scatter(ctx, dC, dA, dB, stage=lambda w: stage_peers(ctx, w, peers))
+    kernel = _lib.last_kernel()
+    assert kernel.startswith("mfma_bf16_256x256"), kernel
+    assert ws.locks.numel() == 2048 and torch.all(ws.locks.cpu() == 1)
+    aux = ws.aux_buffer.cpu()
+    assert oracle.rel_frobenius(aux, oracle.gemm(A, B)) <= 1e-2
+    rows = slice(1024 * rank, 1024 * (rank + 1))
+    assert torch.equal(torch.from_numpy(oracle.owner_map(M, N, 256, 64, W, "reduce_scatter") == rank).nonzero()[:, 0].unique(),
+                       torch.arange(rows.start, rows.stop)), "the rank owns exactly its 1024-row block"
+    got = slot_copies(ctx, dC)
+    want = oracle.slot_sum(aux[rows], [p[rows] for p in peers if p is not None])
+    assert_bits_equal(got[rank][rows], want, f"rank {rank}: slot sum of the owned block from the kernel's own aux")
+    exp = oracle.matmul_reduce_scatter(A, B, peers, rank, W, 256, 64)
+    assert oracle.rel_frobenius(got[rank], exp["C"][rank]) <= 1e-2
+    other = torch.ones(M, dtype=torch.bool)
+    other[rows] = False
+    assert torch.all(got[rank][other] == 0), "rows of other owners are left alone"
+    for r in range(W):
+        if r != rank:
+            assert torch.all(got[r] == 0), f"slot {r} was written"
+
+
 def _fp8_case(M, N, K, W, block_m):
     a, b = randn_cpu((M, K), 0, torch.float32), randn_cpu((K, N), 1, torch.float32)
     Aq, sa = oracle.quantize_e4m3(a)
@@ -134,26 +170,35 @@ def _fp8_case(M, N, K, W, block_m):
     dC = ctx.zeros((M, N), dtype=torch.bfloat16)
     cfg = iris.FusedConfig(block_size_m=block_m, block_size_n=64, block_size_k=64, all_reduce_variant="one_shot")
     ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
-    gen = torch.Generator(device="cuda").manual_seed(5)
-    for r in range(1, W):
-        ctx.peer_view(ws.aux_buffer, r).copy_(torch.randn((M, N), generator=gen, device="cuda").to(torch.bfloat16))
+    for r in range(1, W):  # peers' partial results: bf16 N(0,1) from the CPU generator, seed r
+        ctx.peer_view(ws.aux_buffer, r).copy_(randn_cpu((M, N), r, torch.bfloat16))
         ctx.peer_view(ws.locks, r).fill_(1)
     ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, scale_a=sa, scale_b=sb)
     return ctx, ws, dC, Aq, Bq, sa * sb, _lib.last_kernel()
 
 
 def test_config5a_fp8_matmul_all_reduce():
+    """Every row of the 16384 x 8192 output, in chunks the CPU product finishes in seconds."""
     M, N, K, W = 16384, 8192, 1024, 8
     ctx, ws, dC, Aq, Bq, scale, kernel = _fp8_case(M, N, K, W, 256)
     assert kernel.startswith("mfma_fp8_256x256"), kernel
     assert torch.all(ws.locks.cpu() == 1)
-    for r0 in (0, 5120, M - 256):
-        rows = slice(r0, r0 + 256)
+    err2 = ref2 = 0.0
+    step = 2048
+    for r0 in range(0, M, step):
+        rows = slice(r0, r0 + step)
         own = oracle.gemm(Aq[rows], Bq, torch.bfloat16, scale)
         aux = ws.aux_buffer[rows].cpu()
-        assert oracle.rel_frobenius(aux, own) <= 3e-2
+        assert oracle.rel_frobenius(aux, own) <= 3e-2, f"rows {r0}"
+        err2 += float(((aux.double() - own.double()) ** 2).sum())
+        ref2 += float((own.double() ** 2).sum())
         peers = [ctx.peer_view(ws.aux_buffer, r)[rows].cpu() for r in range(1, W)]
+        if r0 == 0:
+            assert_bits_equal(peers[0], randn_cpu((M, N), 1, torch.bfloat16)[rows], "staged peer 1")
         assert_bits_equal(dC[rows].cpu(), oracle.slot_sum(aux, peers), f"rows {r0}")
+        for r in range(1, W):
+            assert torch.all(ctx.peer_view(dC, r)[rows] == 0), f"one-shot wrote slot {r}"
+    assert (err2 / ref2) ** 0.5 <= 3e-2
 
 
 def test_config5b_fp8_skinny():

@@ -441,6 +441,33 @@ def test_unstaged_peer_flags_time_out():
     assert torch.all(ws.locks.cpu() == 1), "own flags are raised before waiting"
 
 
+def test_heap_tensors_outlive_their_context(monkeypatch):
+    """The heap allocation is released with its last tensor, not with the context object."""
+    from iris_amd.host import hip as hip_mod
+
+    freed = []
+    real_free = hip_mod.hip_free
+    monkeypatch.setattr(hip_mod, "hip_free", lambda ptr: (freed.append(ptr), real_free(ptr)))
+    ctx = _ctx(2)
+    base = ctx.heap.base_address
+    t = ctx.zeros((256, 256), dtype=torch.float32)
+    peer = ctx.peer_view(t, 1)
+    t.fill_(2.0)
+    peer.fill_(5.0)
+    del ctx
+    import gc
+    gc.collect()
+    assert base not in freed
+    assert float(t.sum()) == 2.0 * 256 * 256 and float(peer.sum()) == 5.0 * 256 * 256
+    del t
+    gc.collect()
+    assert base not in freed, "a peer view still holds the heap"
+    del peer
+    gc.collect()
+    torch.cuda.synchronize()
+    assert freed.count(base) == 1
+
+
 def test_c_abi_rejects_bad_arguments():
     lib = _lib.library()
     import ctypes

@@ -281,6 +281,55 @@ def test_library_exports_every_declared_symbol():
     assert _lib.last_error() == ""
 
 
+def test_null_context_tensor_is_rejected_before_any_launch():
+    """Every kernel translates addresses through the heap bases, so a NULL context tensor is an
+    argument error for every fused entry point, whatever the world size; the check comes before the
+    first HIP call (the pointers below are never dereferenced)."""
+    lib = _lib.library()
+    null, p = ctypes.c_void_p(0), ctypes.c_void_p(0x10000)
+    for W in (1, 4):
+        rc = lib.iris_hip_matmul_all_reduce(p, p, p, p, p, 64, 64, 64, 64, 1, 64, 1, 64, 1, null, 0, W, 64, 64, 32,
+                                            _lib.VARIANT_ONE_SHOT, _lib.FP32, _lib.FP32, 1.0, 0, 0, null,
+                                            _lib.PATH_GENERIC, null)
+        assert rc == 1 and "context_tensor" in _lib.last_error()
+        rc = lib.iris_hip_matmul_all_reduce(p, p, p, null, null, 64, 64, 64, 64, 1, 64, 1, 64, 1, null, 0, W, 64, 64, 32,
+                                            _lib.VARIANT_ATOMIC, _lib.BF16, _lib.BF16, 1.0, 0, 0, null, 0, null)
+        assert rc == 1 and "context_tensor" in _lib.last_error()
+        rc = lib.iris_hip_matmul_reduce_scatter(p, p, p, p, p, 64, 64, 64, 64, 1, 64, 1, 64, 1, null, 0, W, 64, 64, 32,
+                                                0, 1, _lib.BF16, _lib.BF16, 1.0, 0, 0, null, 0, null)
+        assert rc == 1 and "context_tensor" in _lib.last_error()
+        rc = lib.iris_hip_all_gather_matmul(p, p, p, null, 64, 64, 64 * W, 64, 64, 1, 64, 1, 64, 1, 1, null, 0, W,
+                                            64, 64, 32, _lib.GATHER_K, _lib.BF16, _lib.BF16, _lib.BF16, 1.0, 0, null)
+        assert rc == 1 and "context_tensor" in _lib.last_error()
+        rc = lib.iris_hip_matmul_all_gather(p, p, p, null, 64, 64 * W, 64, 64, 64, 1, 64, 1, 64, 1, 1, null, 0, W,
+                                            64, 64, 32, _lib.BF16, _lib.BF16, _lib.BF16, 1.0, 0, null)
+        assert rc == 1 and "context_tensor" in _lib.last_error()
+
+
+def test_device_span_releases_its_memory_exactly_once():
+    """The object torch keeps alive for the heap's tensors owns the allocation."""
+    from iris_amd.host.heap import _DeviceSpan
+
+    freed = []
+    span = _DeviceSpan(0x7000, 64, freed.append)
+    assert span.__cuda_array_interface__["data"] == (0x7000, False)
+    keeper = span  # a second reference, as torch's tensor storage holds one
+    del span
+    assert freed == []
+    del keeper
+    assert freed == [0x7000]
+    _DeviceSpan(0x7000, 64)  # no release callback: nothing to do
+    assert freed == [0x7000]
+
+
+def test_host_heap_tensors_outlive_their_context():
+    ctx = cpu_ctx()
+    t = ctx.zeros((8, 8), dtype=torch.float32)
+    t.fill_(3.0)
+    del ctx
+    assert float(t.sum()) == 192.0
+
+
 def test_header_enumerations_match_python():
     header = open(os.path.join(ROOT, "include", "iris_hip.h")).read()
     values = {k: int(v) for k, v in re.findall(r"(IRIS_HIP_[A-Z0-9_]+)\s*=\s*(\d+)", header)}
