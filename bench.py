@@ -1,15 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the rank-local fused GEMM+collective path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--protocol both|flushed|back_to_back]
 
 Prints ONE JSON line.  A step is one launch of the fused operator on synthetic inputs that already
-sit in HBM (peers' partial results and flags staged before the timed region).  `value` is the
-whole-job throughput of the K timed steps in TFLOP/s (2*M*N*K flop per step); `roofline` prices the
-same launches, timed one by one with GPU events on the launch stream, against the roof that bounds
-the fused kernel (HBM for the slot-sum workloads, MFMA for the others); `gemm_phase` repeats the
-measurement with the peers switched off (W = 1), which isolates the MFMA phase; `cpu_baseline` times
-torch's CPU matmul plus the slot reduction on a bounded sample of the same workload.
+sit in HBM (peers' partial results and flags staged before the timed region).
+
+Two timing passes:
+  * back to back: W untimed steps, then K timed steps between two device synchronisations; `value` is
+    the whole-job throughput of those K steps in TFLOP/s (2*M*N*K flop per step, wall clock).
+  * flushed, the protocol of the reference's iris.do_bench (iris/host/platform/utils.py:137-201):
+    before every launch the device is synchronised, a 256 MB buffer is zeroed to push the previous
+    launch's lines out of L2 / last-level cache, the device is synchronised again, and the launch is
+    bracketed by GPU events on the launch stream; 25 warm-up and 100 timed launches, mean and median.
+`roofline` prices the flushed launches against the roof that bounds the fused kernel (HBM for the
+slot-sum workloads, MFMA for the others) and also carries the back-to-back per-launch figures;
+`gemm_phase` repeats the measurement with the peers switched off (W = 1), which isolates the MFMA
+phase; `cpu_baseline` times torch's CPU matmul plus the slot reduction on the same workload.
 
 Default workload: the headline configuration, matmul_all_reduce bf16 M=N=4096, K=1376, W=8.
 """
@@ -70,8 +77,16 @@ class MatmulAllReduce(Workload):
         self.flops = 2 * M * N * K
 
     def algorithmic_bytes(self, world):
+        """Compulsory HBM traffic of one launch: A, B, the peers' tiles this rank reduces, the stores
+        of the reduced tiles.  one_shot reduces every tile into the own C; a two_shot rank reduces the
+        1/W of the tiles it owns and stores each of them into all W slots.  The aux round trip and the
+        flags are not counted."""
         es = 1 if self.fp8 else 2
-        return self.M * self.K * es + self.K * self.N * es + (world - 1) * self.M * self.N * 2 + self.M * self.N * 2
+        mn = self.M * self.N * 2
+        ab = self.M * self.K * es + self.K * self.N * es
+        if self.variant == "two_shot":
+            return ab + (world - 1) * mn // world + world * (mn // world)
+        return ab + (world - 1) * mn + mn
 
     def describe(self, world):
         return {"workload": self.name, "op": "matmul_all_reduce", "variant": self.variant, "M": self.M, "N": self.N,
@@ -101,10 +116,8 @@ class MatmulAllReduce(Workload):
         self.cfg = iris.FusedConfig(block_size_m=self.block_m, block_size_n=64, block_size_k=64,
                                     all_reduce_variant=self.variant)
         self.ws = ops.matmul_all_reduce_preamble(ctx, self.C, self.A, self.B, config=self.cfg)
-        gen = torch.Generator(device="cuda").manual_seed(1)
-        for r in range(1, world):  # synthetic peer partials, N(0,1) in bf16, flags raised
-            ctx.peer_view(self.ws.aux_buffer, r).copy_(
-                torch.randn((M, N), generator=gen, device="cuda", dtype=torch.float32).to(self.elem))
+        for r in range(1, world):  # synthetic peer partials: N(0,1) from the CPU generator, seed r; flags raised
+            ctx.peer_view(self.ws.aux_buffer, r).copy_(_randn((M, N), r, self.elem))
             ctx.peer_view(self.ws.locks, r).fill_(1)
         self._op = ops.matmul_all_reduce
         torch.cuda.synchronize()
@@ -115,31 +128,25 @@ class MatmulAllReduce(Workload):
         self._op(self.ctx, self.C, self.A, self.B, async_op=True, config=self.cfg, workspace=self.ws, **self.scale)
 
     def cpu_baseline(self, world, budget_s=20.0):
-        """torch CPU matmul (bf16 in, as the GPU path; fp8 dequantised to fp32) + slot reduction, on
-        the first rows of the workload."""
-        rows = min(self.M, 1024)
+        """torch CPU matmul (bf16 in, as the GPU path; fp8 dequantised to fp32) + slot reduction with
+        the same seeded peers, on the whole workload when one pass costs well under a second of CPU
+        time, else on its first 2048 rows."""
+        rows = self.M if self.flops <= 1e11 else min(self.M, 2048)
         A = self.A_cpu[:rows]
         A = A.float() if self.fp8 else A
         B = self.B_cpu.float() if self.fp8 else self.B_cpu
-        peers = [_randn((rows, self.N), 100 + r, torch.bfloat16) for r in range(1, world)]
+        peers = [_randn((self.M, self.N), r, self.elem)[:rows].contiguous() for r in range(1, world)]
 
         def once():
-            C = torch.matmul(A, B).to(torch.bfloat16)
+            C = torch.matmul(A, B).to(self.elem)
             acc = C.float()
             for p in peers:
                 acc += p.float()
-            return acc.to(torch.bfloat16)
+            return acc.to(self.elem)
 
-        once()
-        times, t_end = [], time.perf_counter() + budget_s
-        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
-            t0 = time.perf_counter()
-            once()
-            times.append(time.perf_counter() - t0)
-        t = statistics.median(times)
-        return {"value": 2 * rows * self.N * self.K / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-                "kind": "port", "sample": f"first {rows} of {self.M} rows, {len(times)} reps, median; "
-                                          f"torch.matmul + fp32 sum of {world} slots; os.cpu_count={os.cpu_count()}"}
+        which = "all" if rows == self.M else "first"
+        return _time_cpu(once, 2 * rows * self.N * self.K, budget_s,
+                         f"{which} {rows} of {self.M} rows; torch.matmul + fp32 sum of {world} slots")
 
 
 class AllGatherMatmul(Workload):
@@ -188,18 +195,26 @@ class AllGatherMatmul(Workload):
 
 
 class MatmulReduceScatter(Workload):
+    """accumulate=False: one launch stands in for every rank's reduce step (row block r lands in slot r,
+    peers contribute nothing).  accumulate=True: the reference semantics for rank 0 - seven staged peer
+    aux buffers, the rank's own row block summed over the slots in fp32 and stored to its C."""
+
     bound = "bf16"
 
-    def __init__(self, name, M, N, K):
-        self.name, self.M, self.N, self.K = name, M, N, K
+    def __init__(self, name, M, N, K, accumulate=False):
+        self.name, self.M, self.N, self.K, self.accumulate = name, M, N, K, accumulate
         self.flops = 2 * M * N * K
 
     def algorithmic_bytes(self, world):
-        return 2 * (self.M * self.K + self.K * self.N + self.M * self.N)
+        ab = 2 * (self.M * self.K + self.K * self.N)
+        mn = 2 * self.M * self.N
+        if self.accumulate:  # the owned 1/W of the output: W-1 peer blocks read, one block written
+            return ab + (world - 1) * (mn // world) + mn // world
+        return ab + mn
 
     def describe(self, world):
         return {"workload": self.name, "op": "matmul_reduce_scatter", "M": self.M, "N": self.N, "K": self.K,
-                "W": world, "all_owners": True, "sum_peers": False}
+                "W": world, "all_owners": not self.accumulate, "sum_peers": self.accumulate}
 
     def setup(self, iris, world):
         from iris_amd import _lib
@@ -215,7 +230,12 @@ class MatmulReduceScatter(Workload):
         self.C = ctx.zeros((M, N), dtype=torch.bfloat16)
         cfg = FusedConfig()
         ws = matmul_reduce_scatter_preamble(ctx, self.C, self.A, self.B, cfg)
+        if self.accumulate:
+            for r in range(1, world):  # peers' partial products: bf16 N(0,1), CPU generator, seed r
+                ctx.peer_view(ws.aux_buffer, r).copy_(_randn((M, N), r, torch.bfloat16))
+                ctx.peer_view(ws.locks, r).fill_(1)
         A, B, C = self.A, self.B, self.C
+        all_owners, sum_peers = (0, 1) if self.accumulate else (1, 0)
         # The operator wrapper re-runs its preamble (two barriers, three memsets) on every call, as
         # the reference does; the step times the launch alone, through the same C entry point.
         self._launch = lambda: iris_launch(
@@ -223,8 +243,8 @@ class MatmulReduceScatter(Workload):
             ptr(A), ptr(B), ptr(C), ptr(ws.aux_buffer), ptr(ws.locks), M, N, K,
             A.stride(0), A.stride(1), B.stride(0), B.stride(1), C.stride(0), C.stride(1),
             ptr(ctx.get_device_context()), 0, world, cfg.block_size_m, cfg.block_size_n, cfg.block_size_k,
-            1, 0, _lib.BF16, _lib.BF16, 1.0, _lib.ACC_FP32, ctx.spin_limit, ptr(ctx._status), _lib.PATH_AUTO,
-            current_stream(ctx), algorithm="matmul_reduce_scatter", rank=0)
+            all_owners, sum_peers, _lib.BF16, _lib.BF16, 1.0, _lib.ACC_FP32, ctx.spin_limit, ptr(ctx._status),
+            _lib.PATH_AUTO, current_stream(ctx), algorithm="matmul_reduce_scatter", rank=0)
         torch.cuda.synchronize()
 
     def step(self):
@@ -325,6 +345,8 @@ WORKLOADS = {
     "all_gather_matmul_bf16_8192x1792x4096": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096", 8192, 1792, 4096),
     "all_gather_matmul_bf16_8192x1792x4096_nt": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096_nt", 8192, 1792, 4096, b_transposed=True),
     "matmul_reduce_scatter_bf16_8192x4096x1376": lambda: MatmulReduceScatter("matmul_reduce_scatter_bf16_8192x4096x1376", 8192, 4096, 1376),
+    "matmul_reduce_scatter_accumulate_bf16_8192x4096x1376": lambda: MatmulReduceScatter(
+        "matmul_reduce_scatter_accumulate_bf16_8192x4096x1376", 8192, 4096, 1376, accumulate=True),
     "matmul_all_reduce_fp8_16384x8192x1024": lambda: MatmulAllReduce("matmul_all_reduce_fp8_16384x8192x1024", 16384, 8192, 1024, fp8=True),
     "matmul_all_reduce_fp8_skinny_32x8192x1024": lambda: MatmulAllReduce(
         "matmul_all_reduce_fp8_skinny_32x8192x1024", 32, 8192, 1024, fp8=True, block_m=32),
@@ -398,6 +420,48 @@ def timed_steps(wl, steps, warmup, graph=False):
     return wall, per_launch_ms
 
 
+FLUSH_BYTES = int(256e6)
+
+
+def flushed_launches(wl, n_warmup=25, n_repeat=100):
+    """Per-launch GPU-event times in ms under the protocol of the reference's do_bench
+    (iris/host/platform/utils.py:137-201): synchronise, zero a 256 MB buffer, synchronise, then the
+    launch alone between two events.  Warm-up launches go through the same sequence."""
+    cache = torch.empty(FLUSH_BYTES // 4, dtype=torch.int, device="cuda")
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    for i in range(-n_warmup, n_repeat):
+        torch.cuda.synchronize()
+        cache.zero_()
+        torch.cuda.synchronize()
+        if i < 0:
+            wl.step()
+            continue
+        starts[i].record()
+        wl.step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wl.ctx.check_status()
+    del cache
+    return [s.elapsed_time(e) for s, e in zip(starts, ends)]
+
+
+def measure(wl, args):
+    """Both timing passes for one prepared workload.  Returns (wall seconds of the K back-to-back
+    steps or None, back-to-back per-launch ms or None, flushed per-launch ms or None)."""
+    wall = b2b = flushed = None
+    if args.protocol in ("both", "back_to_back"):
+        wall, b2b = timed_steps(wl, args.steps, args.warmup, args.graph)
+    if args.protocol in ("both", "flushed"):
+        flushed = flushed_launches(wl)
+    return wall, b2b, flushed
+
+
+def _stats(ms):
+    return None if ms is None else {"mean": round(statistics.mean(ms), 5), "median": round(statistics.median(ms), 5),
+                                    "min": round(min(ms), 5), "n": len(ms)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -405,6 +469,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--world", type=int, default=8, help="number of heap slots W")
+    ap.add_argument("--protocol", default="both", choices=["both", "flushed", "back_to_back"],
+                    help="timing passes to run: K back-to-back steps (value), cache-flushed launches (roofline), or both")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm-phase", action="store_true", help="skip the W=1 measurement")
     ap.add_argument("--graph", action="store_true", help="capture the K steps into one HIP graph and time its replay")
@@ -420,11 +486,17 @@ def main():
 
     wl = WORKLOADS[args.workload]()
     wl.setup(iris, args.world)
-    wall, per_launch_ms = timed_steps(wl, args.steps, args.warmup, args.graph)
+    wall, b2b, flushed = measure(wl, args)
     kernel = _lib.last_kernel() if not isinstance(wl, CopyCalibration) else "torch copy kernel"
-    ms_per_step = wall * 1e3 / args.steps
-    launch_ms = statistics.mean(per_launch_ms)
-    tflops = wl.flops * args.steps / wall / 1e12
+    # The roofline prices the flushed launches (the back-to-back ones when only those were run).
+    priced = flushed if flushed is not None else b2b
+    launch_ms = statistics.mean(priced)
+    if wall is not None:
+        ms_per_step = wall * 1e3 / args.steps
+        tflops = wl.flops * args.steps / wall / 1e12
+    else:  # flushed launches only: no back-to-back region, the value is per launch
+        ms_per_step = launch_ms
+        tflops = wl.flops / (launch_ms * 1e-3) / 1e12
 
     bytes_alg = wl.algorithmic_bytes(args.world)
     if wl.bound == "hbm":
@@ -435,8 +507,9 @@ def main():
         achieved = wl.flops / (launch_ms * 1e-3) / 1e12
     roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "achieved": round(achieved, 2), "peak": peak,
                 "unit": unit, "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload, args.world),
-                "kernel": kernel,
-                "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(per_launch_ms), 5),
+                "kernel": kernel, "flushed": flushed is not None,
+                "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(priced), 5),
+                "launch_ms_flushed": _stats(flushed), "launch_ms_back_to_back": _stats(b2b),
                 "algorithmic_bytes": bytes_alg, "algorithmic_flops": wl.flops}
 
     out = {
@@ -452,7 +525,7 @@ def main():
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
-        "launch_mode": "hip graph replay" if args.graph else "eager",
+        "launch_mode": ("hip graph replay" if args.graph else "eager") if wall is not None else "flushed launches only",
         "config": wl.describe(args.world),
         "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2) if wl.dtype in PEAK else None,
         "roofline": roofline,
@@ -462,11 +535,17 @@ def main():
         del wl.ctx, wl
         torch.cuda.empty_cache()
         solo = WORKLOADS[args.workload]()
-        solo.setup(iris, 1)  # W = 1: same kernel and shape, no peers to sum
-        wall1, per1 = timed_steps(solo, args.steps, args.warmup, args.graph)
-        t1 = solo.flops * args.steps / wall1 / 1e12
-        out["gemm_phase"] = {"world": 1, "tflops": round(t1, 3), "ms_per_step": round(wall1 * 1e3 / args.steps, 5),
-                             "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4), "kernel": _lib.last_kernel()}
+        solo.setup(iris, 1)  # W = 1: same kernel and shape (aux, flags and C still written), no peers to sum
+        wall1, b2b1, flushed1 = measure(solo, args)
+        priced1 = flushed1 if flushed1 is not None else b2b1
+        t1 = solo.flops / (statistics.mean(priced1) * 1e-3) / 1e12  # per launch, like the roofline
+        gp = {"world": 1, "tflops": round(t1, 3), "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4),
+              "flushed": flushed1 is not None, "launch_ms_flushed": _stats(flushed1),
+              "launch_ms_back_to_back": _stats(b2b1), "kernel": _lib.last_kernel()}
+        if wall1 is not None:
+            gp["ms_per_step"] = round(wall1 * 1e3 / args.steps, 5)
+            gp["tflops_per_step_wall"] = round(solo.flops * args.steps / wall1 / 1e12, 3)
+        out["gemm_phase"] = gp
         wl = solo
 
     if not args.no_cpu:
