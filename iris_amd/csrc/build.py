@@ -55,25 +55,35 @@ def _run(cmd, verbose):
         print(out)
 
 
-def build(force=True, verbose=True):
-    """Compile the library.  With force=False an up-to-date library is left alone."""
+STAMPS_OUTPUT = os.path.join(os.path.dirname(HERE), "lib", "libiris_hip_stamps.so")
+
+
+def build(force=True, verbose=True, stamps=False):
+    """Compile the library.  With force=False an up-to-date library is left alone.  stamps=True builds
+    the diagnostic variant (kernels record time stamps at their phase boundaries; see
+    iris_amd/bench/phase_stamps.py) as libiris_hip_stamps.so next to the regular library."""
+    if stamps:
+        return _build(STAMPS_OUTPUT, FLAGS + ["-DIRIS_HIP_PHASE_STAMPS"], verbose)
     if not force and up_to_date():
         return OUTPUT
+    return _build(OUTPUT, FLAGS, verbose)
+
+
+def _build(output, flags, verbose):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    os.makedirs(os.path.dirname(OUTPUT), exist_ok=True)
+    os.makedirs(os.path.dirname(output), exist_ok=True)
     with tempfile.TemporaryDirectory(prefix="iris_hip_build_") as tmpdir:
         objects = [os.path.join(tmpdir, os.path.splitext(os.path.basename(src))[0] + ".o") for src in SOURCES]
         with concurrent.futures.ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
-            jobs = [pool.submit(_run, [hipcc] + FLAGS + ["-c", "-o", obj, src], verbose)
+            jobs = [pool.submit(_run, [hipcc] + flags + ["-c", "-o", obj, src], verbose)
                     for src, obj in zip(SOURCES, objects)]
             for job in jobs:
                 job.result()
-        tmp = OUTPUT + ".tmp"
+        tmp = output + ".tmp"
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp] + objects, verbose)
-        os.replace(tmp, OUTPUT)
-    return OUTPUT
+        os.replace(tmp, output)
+    return output
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv or True)
-    print(OUTPUT)
+    print(build(force=True, stamps="--stamps" in sys.argv))

@@ -63,8 +63,26 @@ struct FusedParams {
   int* status;
   int tiles_m, tiles_n, group_m, num_xcd;
   int row_offset;  // all-gather: first row of this rank's block in the gathered output
-  int stream_peers;  // phase 2 reads the peers' tiles and writes C with non-temporal accesses
+#ifdef IRIS_HIP_PHASE_STAMPS
+  unsigned long long* stamps;  // diagnostic build: 16 time stamps per workgroup (see PHASE_STAMP)
+#endif
 };
+
+// Diagnostic build (-DIRIS_HIP_PHASE_STAMPS): thread 0 of every workgroup records the constant-rate
+// 100 MHz counter at the phase boundaries of its first tile, into p.stamps[blockIdx.x * 16 + i]:
+//   0 kernel entry, 1 first operands in LDS, 2 K loop done, 3 tile staged in LDS, 4 phase-1 stores
+//   issued, 5 phase-1 stores acknowledged, 6 own flags raised and peers' flags seen, 7 phase-2 stores
+//   issued, 8 last store acknowledged.  The regular build compiles the macro away.
+#ifdef IRIS_HIP_PHASE_STAMPS
+#define PHASE_STAMP(i)                                                                         \
+  do {                                                                                         \
+    if (p.stamps && threadIdx.x == 0 && it == 0) p.stamps[blockIdx.x * 16 + (i)] = wall_clock64(); \
+  } while (0)
+#else
+#define PHASE_STAMP(i) \
+  do {                 \
+  } while (0)
+#endif
 
 // ------------------------------------------------------------------------------------------------
 // Small device helpers
@@ -436,6 +454,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   for (int it = 0; ONE_ROUND ? it < 1 : true; ++it) {
     const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
     if (tidx < 0) break;
+    PHASE_STAMP(0);
     int tm, tn;
     grouped_tile(tidx, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
@@ -533,6 +552,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     for (int s = 0; s < AHEAD; ++s) issue(s);
     wait_vmcnt<(AHEAD - 1) * (LA + LB)>();
     __builtin_amdgcn_s_barrier();
+    PHASE_STAMP(1);
     Frags<CFG> fr[KS < 2 ? 2 : KS];  // one set per k-slice (two for the loops that double-buffer)
     if constexpr (!PINGPONG) load_frags(fr[0], 0, 0);
 
@@ -698,6 +718,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     // sure every wave has finished reading operands.
     wait_vmcnt<0>();
     __syncthreads();
+    PHASE_STAMP(2);
 
     // ---- epilogue -------------------------------------------------------------------------------
     // The whole output tile is first written to LDS in the output type (the operand ring is dead
@@ -732,6 +753,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           }
     }
     __syncthreads();
+    PHASE_STAMP(3);
 
     constexpr int CPR = BN / 8;            // 16-byte chunks per tile row
     constexpr int RPP = NT / CPR;          // tile rows covered by one pass of the workgroup
@@ -788,6 +810,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       }
     }
 
+    PHASE_STAMP(4);
     if (flags) {
       // Publish: the aux tile was stored write-through at system scope; every wave waits until its
       // stores are acknowledged, the workgroup meets, and the threads that own flags raise them
@@ -796,11 +819,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // every wave poll and run ahead measured slower.
       wait_vmcnt<0>();
       __syncthreads();
+      PHASE_STAMP(5);
       raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
       if (!solo) {
         wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
         __syncthreads();
       }
+      PHASE_STAMP(6);
 
       // Phase 2: reduce the flag tiles this rank is responsible for.  The peer loads are issued
       // unconditionally (rows this thread does not reduce read the tile origin instead) and for a
@@ -818,9 +843,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       for (int i = 0; i < kMaxCachedSlots - 1; ++i) pb[i] = (i < p.rank ? hb[i] : hb[i + 1]) + (aux_own - hb_own);
       const long long safe_off = ((long long)m0 * p.s_cm + n0) * 2;  // first element of the tile
 
-      auto reduce_tile = [&](auto np_tag, auto nt_tag) {
+      // The peers' tiles are read once and C is written once, so both go past the caches' keep
+      // policy (non-temporal): they neither displace the operands nor - what costs more - make the
+      // last-level cache write back whatever dirty lines it holds to take them in (measured on the
+      // 4096 x 4096 x 1376 bf16 launch with seven peers, after a 256 MB buffer had been zeroed: phase 2
+      // 68 -> 39 us; with the peers' tiles already cached the two policies tie for the one-shot variant).
+      auto reduce_tile = [&](auto np_tag) {
         constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
-        constexpr bool NT = decltype(nt_tag)::value;  // peers' tiles and C bypass the caches' keep policy
         constexpr int NPV = NP > 0 ? NP : 1;
         // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
         // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
@@ -846,8 +875,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
             if constexpr (NP > 0) {
 #pragma unroll
               for (int i = 0; i < NP; ++i) {
-                if constexpr (NT) pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
-                else pv[g][i] = *(const u32x4_t*)(pb[i] + eoff[g]);
+                pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
               }
             }
             own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
@@ -876,7 +904,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
               for (int i = 0; i < NP; ++i) add_peer(pv[g][i]);
             } else if constexpr (NP < 0) {
               for (int pr = 0; pr < p.world; ++pr)
-                if (pr != p.rank) add_peer(*(const u32x4_t*)(in_slot(aux_own, pr) + eoff[g]));
+                if (pr != p.rank) add_peer(__builtin_nontemporal_load((const u32x4_t*)(in_slot(aux_own, pr) + eoff[g])));
             }
             u32x4_t res;
 #pragma unroll
@@ -884,14 +912,12 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
               res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
             if (active[g]) {
               if (p.epi == EPI_TWO_SHOT) {
-                *(u32x4_t*)(c_own + eoff[g]) = res;
+                __builtin_nontemporal_store(res, (u32x4_t*)(c_own + eoff[g]));
                 for (int pr = 0; pr < p.world; ++pr)
-                  if (pr != p.rank) *(u32x4_t*)(in_slot(c_own, pr) + eoff[g]) = res;
+                  if (pr != p.rank) __builtin_nontemporal_store(res, (u32x4_t*)(in_slot(c_own, pr) + eoff[g]));
               } else {
                 const int dst = p.all_owners ? owner[g] : p.rank;
-                u32x4_t* cdst = (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]);
-                if constexpr (NT) __builtin_nontemporal_store(res, cdst);
-                else *cdst = res;
+                __builtin_nontemporal_store(res, (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]));
               }
             }
           }
@@ -899,18 +925,17 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       };
       switch (solo ? -2 : (p.world <= kMaxCachedSlots ? npeers : -1)) {
         case -2: break;  // C was written in phase 1
-        case 1: reduce_tile(std::integral_constant<int, 1>{}, std::false_type{}); break;
-        case 3: reduce_tile(std::integral_constant<int, 3>{}, std::false_type{}); break;
-        case 7:
-          // Peer tiles are read once; when they exceed what the last-level cache holds, streaming
-          // them non-temporally is faster (measured: 663 -> 622 us for 7 x 256 MiB of peers), for
-          // smaller launches it is not (two-shot 4096 x 4096: 91 -> 98 us).
-          if (p.stream_peers) reduce_tile(std::integral_constant<int, 7>{}, std::true_type{});
-          else reduce_tile(std::integral_constant<int, 7>{}, std::false_type{});
-          break;
-        default: reduce_tile(std::integral_constant<int, -1>{}, std::false_type{}); break;
+        case 1: reduce_tile(std::integral_constant<int, 1>{}); break;
+        case 3: reduce_tile(std::integral_constant<int, 3>{}); break;
+        case 7: reduce_tile(std::integral_constant<int, 7>{}); break;
+        default: reduce_tile(std::integral_constant<int, -1>{}); break;
       }
     }
+    PHASE_STAMP(7);
+#ifdef IRIS_HIP_PHASE_STAMPS
+    wait_vmcnt<0>();
+    PHASE_STAMP(8);
+#endif
     // Staging shares LDS with the operand ring of the next tile: every wave must be done reading it.
     // A bare barrier - __syncthreads() would also wait for this tile's global stores to be
     // acknowledged (1-4 us), which nothing here depends on; they drain behind the next tile's

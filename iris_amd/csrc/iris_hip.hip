@@ -316,8 +316,15 @@ extern template int dispatch_mfma_in<IN_FP8>(FusedParams&, int, bool, int, int, 
 
 namespace {
 
+#ifdef IRIS_HIP_PHASE_STAMPS
+unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
+#endif
+
 int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
   g_last_error[0] = 0;
+#ifdef IRIS_HIP_PHASE_STAMPS
+  p.stamps = g_stamps;
+#endif
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("M, N, K must be positive (got %d, %d, %d)", p.M, p.N, p.K);
   if (!p.A || !p.B || !p.C) return fail("A, B and C must not be NULL");
   if (p.world < 1 || p.rank < 0 || p.rank >= p.world) return fail("bad rank/world_size %d/%d", p.rank, p.world);
@@ -354,15 +361,14 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
 
-  p.stream_peers = epi_has_flags(p.epi) && p.sum_peers &&
-                   (long long)(p.world - 1) * p.M * p.N * 2 > (512ll << 20);
   const bool bkc = (p.s_bn != 1);
   switch (in_dtype) {
-    case IRIS_HIP_BF16: return dispatch_mfma_in<IN_BF16>(p, kind, bkc, device, facts->cu_count, s);
-    case IRIS_HIP_FP16: return dispatch_mfma_in<IN_F16>(p, kind, bkc, device, facts->cu_count, s);
-    case IRIS_HIP_FP8_E4M3: return dispatch_mfma_in<IN_FP8>(p, kind, bkc, device, facts->cu_count, s);
+    case IRIS_HIP_BF16: rc = dispatch_mfma_in<IN_BF16>(p, kind, bkc, device, facts->cu_count, s); break;
+    case IRIS_HIP_FP16: rc = dispatch_mfma_in<IN_F16>(p, kind, bkc, device, facts->cu_count, s); break;
+    case IRIS_HIP_FP8_E4M3: rc = dispatch_mfma_in<IN_FP8>(p, kind, bkc, device, facts->cu_count, s); break;
+    default: rc = fail("unsupported input type %d", in_dtype);
   }
-  return fail("unsupported input type %d", in_dtype);
+  return rc;
 }
 
 bool fits_int(int64_t v) { return v > 0 && v < (1ll << 31); }
@@ -522,6 +528,11 @@ int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_
   if (lds_bytes_per_block) *lds_bytes_per_block = f->lds_per_block;
   return 0;
 }
+
+#ifdef IRIS_HIP_PHASE_STAMPS
+// Diagnostic build only: device buffer of 16 x (number of workgroups) 64-bit words, or NULL.
+void iris_hip_debug_set_stamps(void* device_buffer) { g_stamps = (unsigned long long*)device_buffer; }
+#endif
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }
