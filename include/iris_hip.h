@@ -102,6 +102,36 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
                                int64_t spin_limit, int32_t* status, int32_t path, void* stream);
 
 /*
+ * iris_hip_matmul_all_reduce for a single rank (world_size 1: C = cast(A @ B), the reference's own
+ * single-rank test configuration) WITHOUT a caller-provided workspace and without any allocation.
+ *
+ * It has no counterpart in the reference, whose operators always allocate their workspace
+ * (iris/ops/matmul_all_reduce.py:191-219).  It is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The aux buffer, the tile flags and the
+ * one-rank context the kernels need live in a static device array of the library
+ * (IRIS_HIP_NOALLOC_MAX_AUX_BYTES + 64 KiB + 256 bytes on every GPU the library runs on, held until the
+ * process ends).  The call launches a small kernel that clears the flags it is going to use and then the
+ * same kernels as iris_hip_matmul_all_reduce; it calls no hipMalloc / hipFree.
+ *
+ * Limits (hipErrorInvalidValue with a message otherwise): the bytes aux spans with C's strides,
+ * ((M-1)*stride_cm + (N-1)*stride_cn + 1) * sizeof(out element), at most IRIS_HIP_NOALLOC_MAX_AUX_BYTES;
+ * cdiv(M, block_size_m) * cdiv(N, block_size_n) at most IRIS_HIP_NOALLOC_MAX_FLAGS; variant one_shot or
+ * two_shot.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams,
+ * two threads) race on it and must be ordered by the caller.
+ */
+#define IRIS_HIP_NOALLOC_MAX_AUX_BYTES (32 * 1024 * 1024)
+#define IRIS_HIP_NOALLOC_MAX_FLAGS 16384
+int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C,
+                                       int64_t M, int64_t N, int64_t K,
+                                       int64_t stride_am, int64_t stride_ak,
+                                       int64_t stride_bk, int64_t stride_bn,
+                                       int64_t stride_cm, int64_t stride_cn,
+                                       int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                                       int32_t variant,
+                                       int32_t in_dtype, int32_t out_dtype, float scale,
+                                       int32_t path, void* stream);
+
+/*
  * Fused C = reduce_scatter(A @ B), rank-local part.
  * Replaces the launch of _fused_matmul_reduce_scatter_kernel
  * (iris/ops/matmul_reduce_scatter.py:261-288; kernel :25-118; DeviceContext.reduce_scatter

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # IRIS_HIP_LIBRARY names another build of the same library (e.g. one compiled with other tile shapes).
 LIBRARY_PATH = os.environ.get("IRIS_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libiris_hip.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 # Enumerations of include/iris_hip.h
 BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
@@ -21,6 +21,7 @@ GATHER_K, GATHER_M = 1, 2
 PATH_AUTO, PATH_MFMA, PATH_GENERIC = 0, 1, 2
 STATUS_SPIN_TIMEOUT = 1
 DISTRIBUTION_STRIDED, DISTRIBUTION_BLOCK = 0, 1
+NOALLOC_MAX_AUX_BYTES, NOALLOC_MAX_FLAGS = 32 * 1024 * 1024, 16384
 
 _i32, _i64, _f32, _ptr = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -41,6 +42,16 @@ PROTOTYPES = {
         _GEMM_HEAD + [_i32,  # variant
                       _i32, _i32, _f32, _i32,  # in_dtype, out_dtype, scale, acc_mode
                       _i64, _ptr, _i32, _ptr],  # spin_limit, status, path, stream
+    ),
+    "iris_hip_matmul_all_reduce_noalloc": (
+        _i32,
+        [_ptr, _ptr, _ptr,  # A, B, C
+         _i64, _i64, _i64,  # M, N, K
+         _i64, _i64, _i64, _i64, _i64, _i64,  # strides am ak bk bn cm cn
+         _i32, _i32, _i32,  # block sizes m n k
+         _i32,  # variant
+         _i32, _i32, _f32,  # in_dtype, out_dtype, scale
+         _i32, _ptr],  # path, stream
     ),
     "iris_hip_matmul_reduce_scatter": (
         _i32,

@@ -316,6 +316,51 @@ extern template int dispatch_mfma_in<IN_FP8>(FusedParams&, int, bool, int, int, 
 
 namespace {
 
+// ------------------------------------------------------------------------------------------------
+// Library-owned workspace of iris_hip_matmul_all_reduce_noalloc
+// ------------------------------------------------------------------------------------------------
+// Layout of the array: [0, 256) a one-rank context (rank 0, world 1, heap base 0: every address
+// translates to itself), [256, 256 + 64 KiB) the tile flags, then the aux buffer.
+constexpr size_t kScratchContextBytes = 256;
+constexpr size_t kScratchFlagBytes = (size_t)IRIS_HIP_NOALLOC_MAX_FLAGS * sizeof(int32_t);
+constexpr size_t kScratchAuxOffset = kScratchContextBytes + kScratchFlagBytes;
+constexpr size_t kScratchBytes = kScratchAuxOffset + (size_t)IRIS_HIP_NOALLOC_MAX_AUX_BYTES;
+static_assert(kScratchAuxOffset % 256 == 0, "aux buffer alignment");
+
+// Device memory of its own on every GPU the library runs on, from module load to process end.  The
+// name below is a host-side handle only: device code and HIP calls get the address that
+// hipGetSymbolAddress reports for the current device (scratch_for_current_device).
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+void* g_scratch_ptr[64] = {};
+std::mutex g_scratch_mutex;
+
+// Address of the scratch array on the current device (looked up once per device).
+int scratch_for_current_device(unsigned char** out) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return (int)e;
+  if (device < 0 || device >= 64) return fail("device index %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return fail("the library's workspace has no address on device %d", device);
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = (unsigned char*)g_scratch_ptr[device];
+  return 0;
+}
+
+// Writes the one-rank context and clears the flags a launch is going to use.  A kernel, not a memset:
+// the caller's stream may be under graph capture.
+__global__ void __launch_bounds__(256) noalloc_prepare_kernel(long long* context, int* flags, int nflags) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < (int)(kScratchContextBytes / sizeof(long long))) context[i] = (i == 1) ? 1 : 0;  // [rank 0, world 1, base 0, ...]
+  if (i < nflags) flags[i] = 0;
+}
+
 #ifdef IRIS_HIP_PHASE_STAMPS
 unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
 #endif
@@ -430,6 +475,48 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
   return run_fused(p, in_dtype, out_dtype, path, stream);
 }
 
+int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                                       int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                                       int64_t stride_cm, int64_t stride_cn,
+                                       int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                                       int32_t variant, int32_t in_dtype, int32_t out_dtype, float scale,
+                                       int32_t path, void* stream) {
+  g_last_error[0] = 0;
+  if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
+  if (variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
+    return fail("variant %d is not one_shot (2) or two_shot (3)", variant);
+  if (block_size_m <= 0 || block_size_n <= 0) return fail("block sizes must be positive");
+  const int es = elem_size(out_dtype);
+  if (es == 0) return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
+  if (stride_cm < 0 || stride_cn < 0) return fail("negative output strides are not supported");
+  // aux is addressed with C's strides: the bytes it spans and the flags of the tile grid must fit.
+  const long long aux_bytes = ((long long)(M - 1) * stride_cm + (long long)(N - 1) * stride_cn + 1) * es;
+  const long long nflags = (long long)cdiv((int)M, block_size_m) * cdiv((int)N, block_size_n);
+  if (aux_bytes > (long long)IRIS_HIP_NOALLOC_MAX_AUX_BYTES)
+    return fail("output of %lld x %lld spans %lld bytes, beyond the %lld bytes of the library's workspace; "
+                "use iris_hip_matmul_all_reduce with a caller-owned workspace",
+                (long long)M, (long long)N, aux_bytes, (long long)IRIS_HIP_NOALLOC_MAX_AUX_BYTES);
+  if (nflags > IRIS_HIP_NOALLOC_MAX_FLAGS)
+    return fail("%lld tiles of %d x %d, beyond the %d flags of the library's workspace; use larger block sizes "
+                "or iris_hip_matmul_all_reduce with a caller-owned workspace",
+                nflags, block_size_m, block_size_n, IRIS_HIP_NOALLOC_MAX_FLAGS);
+  unsigned char* base = nullptr;
+  int rc = scratch_for_current_device(&base);
+  if (rc) return rc;
+  long long* context = (long long*)base;
+  int32_t* locks = (int32_t*)(base + kScratchContextBytes);
+  void* aux = base + kScratchAuxOffset;
+  const int threads = 256;
+  const int need = (int)nflags > (int)(kScratchContextBytes / sizeof(long long)) ? (int)nflags : (int)(kScratchContextBytes / sizeof(long long));
+  hipLaunchKernelGGL(noalloc_prepare_kernel, dim3((need + threads - 1) / threads), dim3(threads), 0, (hipStream_t)stream,
+                     context, locks, (int)nflags);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  return iris_hip_matmul_all_reduce(A, B, C, aux, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm,
+                                    stride_cn, (const int64_t*)context, 0, 1, block_size_m, block_size_n, block_size_k,
+                                    variant, in_dtype, out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream);
+}
+
 int iris_hip_matmul_reduce_scatter(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
                                    int64_t M, int64_t N, int64_t K,
                                    int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
@@ -526,6 +613,14 @@ int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_
   if (cu_count) *cu_count = f->cu_count;
   if (xcc_count) *xcc_count = f->xcc_count;
   if (lds_bytes_per_block) *lds_bytes_per_block = f->lds_per_block;
+  // Set-up call of the host layer: also look up the no-allocation entry point's workspace address
+  // when `device` is the current one, so that its first call has nothing left to resolve.
+  int current = -1;
+  if (hipGetDevice(&current) == hipSuccess && current == device) {
+    unsigned char* unused = nullptr;
+    rc = scratch_for_current_device(&unused);
+    if (rc) return rc;
+  }
   return 0;
 }
 
@@ -536,6 +631,6 @@ void iris_hip_debug_set_stamps(void* device_buffer) { g_stamps = (unsigned long 
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }
-int iris_hip_abi_version(void) { return 3; }
+int iris_hip_abi_version(void) { return 4; }
 
 }  // extern "C"
