@@ -4,9 +4,14 @@
  *
  * The reference package has no native interface: each operator launches a Triton kernel through
  * `iris_launch(kernel_fn, grid, *args, ...)` (iris/host/tracing/kernel_artifacts.py:54-83).  Every
- * entry point below takes exactly the arguments of one such launch, in the same order and with the
- * same meaning, followed by a short tail of values the Triton launch gets implicitly (element types,
- * the HIP stream) or that this library adds (scales for fp8 inputs, a bound on flag spinning).
+ * entry point below takes the arguments of one such launch, in the same order and with the same
+ * meaning, up to and including the three block sizes, followed by a short tail of values the Triton
+ * launch gets implicitly (element types, the HIP stream) or that this library adds (scales for fp8
+ * inputs, a bound on flag spinning).  The launch arguments after the block sizes are compile-time
+ * tuning constants of the Triton kernels and are NOT taken: EVEN_K everywhere (K tails are handled by
+ * out-of-range loads), and for the two gather operators GROUP_SIZE_M, NUM_SMS, NUM_XCDS,
+ * NUM_K_BLOCKS_LOCAL, USE_BIAS (a NULL bias says the same), EVEN_K and ALLOW_TF32
+ * (iris/ops/all_gather_matmul.py:289-295, iris/ops/matmul_all_gather.py:258-262).
  *
  * Conventions
  *   - All data pointers are device pointers.  Strides are in elements, as torch reports them.
@@ -17,7 +22,10 @@
  *   - Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
  *   - Return value: 0 on success, otherwise a hipError_t value.  Argument errors return
  *     hipErrorInvalidValue (1); iris_hip_last_error() then describes the problem.
- *   - The library allocates no device memory and keeps no state between calls.
+ *   - The library calls no hipMalloc.  It keeps between calls: device facts (CU count, XCD count, LDS
+ *     size) cached per device under a mutex, a once-per-device "attribute set" flag per kernel build
+ *     (atomic), the last error and last kernel name per host thread, and one static device array that
+ *     only iris_hip_matmul_all_reduce_noalloc uses.  Entry points may be called from several host threads.
  */
 #ifndef IRIS_HIP_H
 #define IRIS_HIP_H
