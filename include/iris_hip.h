@@ -24,7 +24,8 @@
  *     hipErrorInvalidValue (1); iris_hip_last_error() then describes the problem.
  *   - The library calls no hipMalloc.  It keeps between calls: device facts (CU count, XCD count, LDS
  *     size) cached per device under a mutex, a once-per-device "attribute set" flag per kernel build
- *     (atomic), the last error and last kernel name per host thread, and one static device array that
+ *     (atomic), the last error and last kernel name per host thread, the contents of context tensors
+ *     registered with iris_hip_register_context (under a mutex), and one static device array that
  *     only iris_hip_matmul_all_reduce_noalloc uses.  Entry points may be called from several host threads.
  */
 #ifndef IRIS_HIP_H
@@ -263,6 +264,20 @@ int iris_hip_reduce_scatter(const void* input, void* output, int64_t M, int64_t 
                             int32_t block_size_m, int32_t block_size_n, int32_t swizzle_size,
                             int32_t comm_sms, int32_t num_xcds, int32_t chunk_size,
                             int32_t distribution, int32_t dtype, void* stream);
+
+/*
+ * Optional: tell the library what a context tensor holds.  `context_tensor` is the device pointer that
+ * later launches pass; `host_copy` points at the same `num_words` int64 words in host memory
+ * ([cur_rank, world_size, heap_base_0 .. heap_base_{W-1}, ...], iris/host/iris.py:916-958).  Launches
+ * that name a registered context tensor (same pointer, rank and world size, at most 8 ranks) get the
+ * heap bases as kernel arguments instead of loading them on the device, which takes a dependent memory
+ * round trip (about 1 us) off the path to the peers' flags and tiles; the decode-sized kernel probes
+ * the peers' flags ahead of its operand loads only then.  Results do not depend on registration.
+ * The contents of a registered tensor must not change, and it must be unregistered before its memory is
+ * freed or reused.  No counterpart in the reference (Triton reads the tensor on the device).
+ */
+int iris_hip_register_context(const int64_t* context_tensor, const int64_t* host_copy, int32_t num_words);
+int iris_hip_unregister_context(const int64_t* context_tensor);
 
 /*
  * Device facts used by the host layer (reference: get_cu_count / get_num_xcc,

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # IRIS_HIP_LIBRARY names another build of the same library (e.g. one compiled with other tile shapes).
 LIBRARY_PATH = os.environ.get("IRIS_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libiris_hip.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 # Enumerations of include/iris_hip.h
 BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
@@ -82,6 +82,8 @@ PROTOTYPES = {
     ),
     "iris_hip_all_reduce": (_i32, _CCL_HEAD + [_i32, _i32, _i32, _ptr]),  # variant, distribution, dtype, stream
     "iris_hip_reduce_scatter": (_i32, _CCL_HEAD + [_i32, _i32, _ptr]),  # distribution, dtype, stream
+    "iris_hip_register_context": (_i32, [_ptr, _ptr, _i32]),
+    "iris_hip_unregister_context": (_i32, [_ptr]),
     "iris_hip_query": (_i32, [_i32, _ptr, _ptr, _ptr]),
     "iris_hip_last_error": (ctypes.c_char_p, []),
     "iris_hip_last_kernel": (ctypes.c_char_p, []),

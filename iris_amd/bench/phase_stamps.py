@@ -101,5 +101,6 @@ def main():
     print(f"  {'first entry -> last stamp':40s} {statistics.mean(spans):8.2f}")
 
 
+
 if __name__ == "__main__":
     main()

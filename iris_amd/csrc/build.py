@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 # compiled side by side), the entry points with the generic kernel, and the stand-alone collectives.
 SOURCES = [os.path.join(HERE, f) for f in (
     "iris_hip.hip", "iris_hip_mfma_bf16.hip", "iris_hip_mfma_f16.hip", "iris_hip_mfma_fp8.hip", "iris_ccl.hip")]
-HEADERS = [os.path.join(HERE, h) for h in ("fused_kernel.h", "layout.h", "device_util.h", "host_common.h")] + [
+HEADERS = [os.path.join(HERE, h) for h in ("fused_kernel.h", "decode_kernel.h", "layout.h", "device_util.h", "host_common.h")] + [
     os.path.join(ROOT, "include", "iris_hip.h")]
 OUTPUT = os.path.join(os.path.dirname(HERE), "lib", "libiris_hip.so")
 

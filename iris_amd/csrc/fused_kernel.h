@@ -63,6 +63,11 @@ struct FusedParams {
   int* status;
   int tiles_m, tiles_n, group_m, num_xcd;
   int row_offset;  // all-gather: first row of this rank's block in the gathered output
+  // Heap bases as kernel arguments (slots 0..7), valid when hb_in_args is set: the host knew the contents
+  // of the context tensor (iris_hip_register_context), which spares the kernels a dependent scalar load
+  // on the way to the peers' flags and tiles.
+  long long hb_arg[8];
+  int hb_in_args;
 #ifdef IRIS_HIP_PHASE_STAMPS
   unsigned long long* stamps;  // diagnostic build: 16 time stamps per workgroup (see PHASE_STAMP)
 #endif
@@ -322,8 +327,16 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   // Heap bases of the first slots, read once (scalar loads) before the kernel stores anything.
   unsigned long long hb[kMaxCachedSlots];
 #pragma unroll
-  for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (p.heap_bases && r < p.world) ? (unsigned long long)p.heap_bases[r] : 0ull;
-  const unsigned long long hb_own = p.heap_bases ? (unsigned long long)p.heap_bases[p.rank] : 0ull;
+  for (int r = 0; r < kMaxCachedSlots; ++r)
+    hb[r] = p.hb_in_args ? (unsigned long long)p.hb_arg[r]
+                         : ((p.heap_bases && r < p.world) ? (unsigned long long)p.heap_bases[r] : 0ull);
+  unsigned long long hb_own = 0ull;
+  if (p.hb_in_args) {
+#pragma unroll
+    for (int r = 0; r < kMaxCachedSlots; ++r) hb_own = (r == p.rank) ? hb[r] : hb_own;
+  } else if (p.heap_bases) {
+    hb_own = (unsigned long long)p.heap_bases[p.rank];
+  }
   auto heap_base = [&](int r) -> unsigned long long {
     unsigned long long v = 0;
     if (r < kMaxCachedSlots) {
@@ -1002,7 +1015,7 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
 //           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
 //           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
 //           tiles the shorter K steps make it the slower of the two.
-enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3 };
+enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
   return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
 }
@@ -1015,12 +1028,20 @@ using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
 template <int IN, bool BKC>
 using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
 
-inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SKINNY ? 64 : 128; }
-inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : 128; }
+inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SKINNY ? 64 : kind == TILE_DECODE ? 32 : 128; }
+inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_DECODE ? 32 : 128; }
+
+#include "decode_kernel.h"
 
 template <int IN>
 int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hipStream_t s) {
   const int bm = tile_rows(kind), bn = tile_cols(kind);
+  if (kind == TILE_DECODE) {
+    static const char* tnames[3] = {"bf16", "f16", "fp8"};
+    char dname[96];
+    snprintf(dname, sizeof(dname), "mfma_%s_32x32x%d_%s", tnames[IN], DecodeCfg<IN, false>::CHUNK, bkc ? "nt" : "nn");
+    return bkc ? launch_decode<IN, true>(p, device, s, dname) : launch_decode<IN, false>(p, device, s, dname);
+  }
   p.tiles_m = cdiv(p.M, bm);
   p.tiles_n = cdiv(p.N, bn);
   // Group height: tile-rows walked together so that an XCD's span of tiles is close to square.

@@ -32,6 +32,7 @@
 
 #include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "fused_kernel.h"
 
@@ -361,6 +362,32 @@ __global__ void __launch_bounds__(256) noalloc_prepare_kernel(long long* context
   if (i < nflags) flags[i] = 0;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Context tensors whose contents the host has told the library (iris_hip_register_context)
+// ------------------------------------------------------------------------------------------------
+struct KnownContext {
+  const int64_t* device_ptr;
+  int rank, world;
+  long long bases[kMaxCachedSlots];
+};
+std::vector<KnownContext> g_contexts;
+std::mutex g_contexts_mutex;
+
+// Fill p.hb_arg from the registry when the launch names a registered context tensor with the same
+// rank and world size (anything else falls back to loading the bases on the device).
+void heap_bases_from_registry(FusedParams& p, const int64_t* context_tensor) {
+  p.hb_in_args = 0;
+  if (!context_tensor || p.world > kMaxCachedSlots) return;
+  std::lock_guard<std::mutex> lock(g_contexts_mutex);
+  for (const KnownContext& k : g_contexts) {
+    if (k.device_ptr != context_tensor) continue;
+    if (k.rank != p.rank || k.world != p.world) return;
+    for (int r = 0; r < kMaxCachedSlots; ++r) p.hb_arg[r] = k.bases[r];
+    p.hb_in_args = 1;
+    return;
+  }
+}
+
 #ifdef IRIS_HIP_PHASE_STAMPS
 unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
 #endif
@@ -382,6 +409,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   }
   // Every kernel translates addresses through the heap bases, also with one rank.
   if (!p.heap_bases) return fail("context_tensor must not be NULL");
+  heap_bases_from_registry(p, (const int64_t*)p.heap_bases - 2);
   if (elem_size(in_dtype) == 0 || elem_size(out_dtype) == 0 || out_dtype == IRIS_HIP_FP8_E4M3)
     return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
 
@@ -396,10 +424,12 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
 
   // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
   // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64-row tiles for decode-sized M, else
-  // 128x128 - two workgroups per CU when there are more such tiles than CUs.
+  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  The flag-carrying operators
+  // with at most 32 rows take the latency-oriented 32x32 kernel (decode_kernel.h).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
+  else if (p.M <= 32 && epi_has_flags(p.epi) && p.gather == GATHER_NONE && p.world <= 8 && !p.bias) kind = TILE_DECODE;
   else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
   const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
@@ -605,6 +635,39 @@ int iris_hip_matmul_all_gather(const void* A, const void* B, void* C_gathered, c
   return run_fused(p, in_dtype, out_dtype, path, stream);
 }
 
+int iris_hip_register_context(const int64_t* context_tensor, const int64_t* host_copy, int32_t num_words) {
+  g_last_error[0] = 0;
+  if (!context_tensor || !host_copy) return fail("context_tensor and host_copy must not be NULL");
+  if (num_words < 3) return fail("a context tensor has at least 3 words (rank, world size, one heap base)");
+  const int64_t rank = host_copy[0], world = host_copy[1];
+  if (world < 1 || rank < 0 || rank >= world || num_words < 2 + world)
+    return fail("bad context contents: rank %lld, world size %lld, %d words", (long long)rank, (long long)world, num_words);
+  KnownContext k;
+  k.device_ptr = context_tensor;
+  k.rank = (int)rank;
+  k.world = (int)world;
+  for (int r = 0; r < kMaxCachedSlots; ++r) k.bases[r] = r < world ? (long long)host_copy[2 + r] : 0ll;
+  std::lock_guard<std::mutex> lock(g_contexts_mutex);
+  for (KnownContext& e : g_contexts)
+    if (e.device_ptr == context_tensor) {
+      e = k;
+      return 0;
+    }
+  g_contexts.push_back(k);
+  return 0;
+}
+
+int iris_hip_unregister_context(const int64_t* context_tensor) {
+  g_last_error[0] = 0;
+  std::lock_guard<std::mutex> lock(g_contexts_mutex);
+  for (size_t i = 0; i < g_contexts.size(); ++i)
+    if (g_contexts[i].device_ptr == context_tensor) {
+      g_contexts.erase(g_contexts.begin() + i);
+      break;
+    }
+  return 0;
+}
+
 int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_t* lds_bytes_per_block) {
   g_last_error[0] = 0;
   DeviceFacts* f = nullptr;
@@ -631,6 +694,6 @@ void iris_hip_debug_set_stamps(void* device_buffer) { g_stamps = (unsigned long 
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }
-int iris_hip_abi_version(void) { return 4; }
+int iris_hip_abi_version(void) { return 5; }
 
 }  // extern "C"

@@ -8,6 +8,7 @@ or the environment (IRIS_NUM_RANKS, IRIS_RANK), falling back to torch.distribute
 initialised, else to a world of one.  All W heaps are slots of one GPU allocation.
 """
 
+import ctypes
 import logging
 import os
 
@@ -98,6 +99,7 @@ class Iris:
 
     def __del__(self):
         try:
+            self._forget_device_context()
             if hasattr(self, "heap"):
                 self.heap.close()
         except Exception:
@@ -235,7 +237,24 @@ class Iris:
 
     def _build_device_context(self):
         data = [self.cur_rank, self.num_ranks] + self.heap_bases.tolist() + [0] * _TRACE_WORDS
-        self._device_context = torch.tensor(data, dtype=torch.int64).to(self.heap.device)
+        host = torch.tensor(data, dtype=torch.int64)
+        self._device_context = host.to(self.heap.device)
+        self._context_registered = False
+        if self.heap.device.type == "cuda" and os.environ.get("IRIS_REGISTER_CONTEXT", "1") != "0":
+            # The kernel library takes the heap bases as kernel arguments when it knows what the
+            # context tensor holds (one dependent load less on the way to the peers' flags).
+            from .. import _lib
+
+            err = _lib.library().iris_hip_register_context(ctypes.c_void_p(self._device_context.data_ptr()),
+                                                           ctypes.c_void_p(host.data_ptr()), host.numel())
+            self._context_registered = err == 0
+
+    def _forget_device_context(self):
+        if getattr(self, "_context_registered", False):
+            from .. import _lib
+
+            _lib.library().iris_hip_unregister_context(ctypes.c_void_p(self._device_context.data_ptr()))
+            self._context_registered = False
 
     def get_device_context(self):
         """int64 tensor [cur_rank, W, heap_base_0..heap_base_{W-1}, 0 x 17] on the Iris device."""

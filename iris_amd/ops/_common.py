@@ -61,7 +61,9 @@ def ptr(t):
 
 
 def current_stream(shmem):
-    return ctypes.c_void_p(torch.cuda.current_stream(shmem.get_device()).cuda_stream)
+    """The raw HIP stream torch would launch on for the context's device right now (honours
+    `with torch.cuda.stream(...)` and graph capture)."""
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(shmem.get_device_id()))
 
 
 def iris_launch(entry_name, grid, *args, algorithm, rank, dtype=None):

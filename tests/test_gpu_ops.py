@@ -557,9 +557,9 @@ def test_ragged_shapes_mfma(M, N, K, variant):
 
 
 # Tile counts that are not a multiple of the eight XCDs and fit in one round: the launch grid is rounded
-# up and the surplus workgroups must find no tile (23 tiles of 64x128 and of 128x128, 27 of 128x128,
-# 140 of 256x256).
-@pytest.mark.parametrize("M,N,K,tile", [(32, 2880, 64, "64x128"), (96, 2880, 64, "128x128"),
+# up and the surplus workgroups must find no tile (90 tiles of 32x32, 23 of 64x128 and of 128x128, 27 of
+# 128x128, 140 of 256x256).
+@pytest.mark.parametrize("M,N,K,tile", [(32, 2880, 64, "32x32"), (48, 2880, 64, "64x128"), (96, 2880, 64, "128x128"),
                                         (384, 1152, 96, "128x128"), (2560, 3584, 64, "256x256")])
 def test_tile_counts_off_the_xcd_multiple(M, N, K, tile):
     W, rank, dtype = 2, 1, torch.float16
