@@ -61,20 +61,6 @@ struct DecodeCfg {
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
-// A copy of the kernel's argument block with every field the kernels read materialised in registers at
-// this point: the empty asm statements use the values, so their loads are issued together, up front.
-__device__ __forceinline__ FusedParams pin_kernel_arguments(const FusedParams& a) {
-  FusedParams q = a;
-  asm volatile("" : "+s"(q.A), "+s"(q.B), "+s"(q.C), "+s"(q.aux), "+s"(q.locks), "+s"(q.heap_bases), "+s"(q.status),
-               "+s"(q.spin_limit), "+s"(q.s_am), "+s"(q.s_bk), "+s"(q.s_bn), "+s"(q.s_cm));
-  asm volatile("" : "+s"(q.M), "+s"(q.N), "+s"(q.K), "+s"(q.rank), "+s"(q.world), "+s"(q.flag_bm), "+s"(q.flag_bn),
-               "+s"(q.epi), "+s"(q.acc_mode), "+s"(q.all_owners), "+s"(q.sum_peers), "+s"(q.scale), "+s"(q.tiles_n),
-               "+s"(q.num_xcd), "+s"(q.hb_in_args));
-  asm volatile("" : "+s"(q.hb_arg[0]), "+s"(q.hb_arg[1]), "+s"(q.hb_arg[2]), "+s"(q.hb_arg[3]), "+s"(q.hb_arg[4]),
-               "+s"(q.hb_arg[5]), "+s"(q.hb_arg[6]), "+s"(q.hb_arg[7]));
-  return q;
-}
-
 // 4-byte direct-to-LDS load at system scope: lane l deposits its dword at lds_base + 4*l (zero when out
 // of range).
 __device__ __forceinline__ void dma4(i32x4_t rsrc, unsigned lds_base, unsigned voff) {
@@ -132,6 +118,8 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
 #pragma unroll
     for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (unsigned long long)p.heap_bases[min(r, p.world - 1)];
   }
+#pragma unroll
+  for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = uniform64(hb[r]);  // scalar registers, whichever branch ran
   unsigned long long hb_own = 0ull;
 #pragma unroll
   for (int r = 0; r < kMaxCachedSlots; ++r) hb_own = (r == p.rank) ? hb[r] : hb_own;

@@ -302,6 +302,45 @@ __device__ __forceinline__ f32x16_t mfma_block(const i32x4_t (&a)[NF], const i32
 
 constexpr int kMaxCachedSlots = 8;  // heap bases kept in registers; larger worlds re-load them
 
+// A 64-bit value that is the same in every lane, moved to scalar registers.
+__device__ __forceinline__ unsigned long long uniform64(unsigned long long x) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)x), hi = __builtin_amdgcn_readfirstlane((unsigned)(x >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// A copy of the kernel's argument block with every field materialised in registers at this point: the
+// empty asm statements use the values, so their loads are issued together, up front.  Left to itself the
+// compiler loads each field next to its first use and waits for it there, which put some twenty
+// dependent scalar round trips in front of the first operand load of a launch.
+__device__ __forceinline__ FusedParams pin_kernel_arguments(const FusedParams& a) {
+  FusedParams q = a;
+  asm volatile("" : "+s"(q.A), "+s"(q.B), "+s"(q.C), "+s"(q.aux), "+s"(q.locks), "+s"(q.bias), "+s"(q.heap_bases),
+               "+s"(q.status), "+s"(q.spin_limit));
+  asm volatile("" : "+s"(q.s_am), "+s"(q.s_ak), "+s"(q.s_bk), "+s"(q.s_bn), "+s"(q.s_cm), "+s"(q.s_cn), "+s"(q.s_bias));
+  asm volatile("" : "+s"(q.M), "+s"(q.N), "+s"(q.K), "+s"(q.K_local), "+s"(q.M_local), "+s"(q.gather), "+s"(q.rank),
+               "+s"(q.world), "+s"(q.flag_bm), "+s"(q.flag_bn), "+s"(q.epi), "+s"(q.acc_mode), "+s"(q.all_owners),
+               "+s"(q.sum_peers), "+s"(q.bias_dtype), "+s"(q.scale));
+  asm volatile("" : "+s"(q.tiles_m), "+s"(q.tiles_n), "+s"(q.group_m), "+s"(q.num_xcd), "+s"(q.row_offset),
+               "+s"(q.hb_in_args));
+  asm volatile("" : "+s"(q.hb_arg[0]), "+s"(q.hb_arg[1]), "+s"(q.hb_arg[2]), "+s"(q.hb_arg[3]), "+s"(q.hb_arg[4]),
+               "+s"(q.hb_arg[5]), "+s"(q.hb_arg[6]), "+s"(q.hb_arg[7]));
+#ifdef IRIS_HIP_PHASE_STAMPS
+  asm volatile("" : "+s"(q.stamps));
+#endif
+  return q;
+}
+
+// The same for the tiled kernel, limited to what it needs before its first operand load (it has no
+// registers to spare for holding the epilogue's arguments across the K loop).
+__device__ __forceinline__ FusedParams pin_loader_arguments(const FusedParams& a) {
+  FusedParams q = a;
+  asm volatile("" : "+s"(q.A), "+s"(q.B), "+s"(q.s_am), "+s"(q.s_bk), "+s"(q.s_bn), "+s"(q.M), "+s"(q.N), "+s"(q.K),
+               "+s"(q.K_local), "+s"(q.M_local), "+s"(q.gather), "+s"(q.rank), "+s"(q.world), "+s"(q.tiles_m),
+               "+s"(q.tiles_n), "+s"(q.group_m), "+s"(q.num_xcd));
+  return q;
+}
+
+
 // ------------------------------------------------------------------------------------------------
 // MFMA kernel
 // ------------------------------------------------------------------------------------------------
@@ -309,7 +348,7 @@ constexpr int kMaxCachedSlots = 8;  // heap bases kept in registers; larger worl
 // tile loop is then known to run once, which lets the compiler drop everything it otherwise carries
 // from tile to tile (measured: 1.2 us of a 9 us launch on decode-sized problems).
 template <class CFG, bool ONE_ROUND>
-__global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kernel(const FusedParams p) {
+__global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kernel(const FusedParams p_in) {
   using Out = typename OutOf<CFG::IN>::type;
   using ATile = RowTile<CFG::RBA>;
   constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
@@ -319,6 +358,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
+  const FusedParams q_args = pin_loader_arguments(p_in);  // the loaders' kernel arguments, fetched in one batch
+  const FusedParams& p = q_args;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -326,16 +367,24 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 
   // Heap bases of the first slots, read once (scalar loads) before the kernel stores anything.
   unsigned long long hb[kMaxCachedSlots];
+  if (p.hb_in_args) {  // kernel arguments when the host knew them
 #pragma unroll
-  for (int r = 0; r < kMaxCachedSlots; ++r)
-    hb[r] = p.hb_in_args ? (unsigned long long)p.hb_arg[r]
-                         : ((p.heap_bases && r < p.world) ? (unsigned long long)p.heap_bases[r] : 0ull);
+    for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (unsigned long long)p.hb_arg[r];
+  } else if (p.heap_bases) {  // else independent loads behind one branch (indices clamped to the world size)
+#pragma unroll
+    for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = (unsigned long long)p.heap_bases[min(r, p.world - 1)];
+  } else {
+#pragma unroll
+    for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = 0ull;
+  }
+#pragma unroll
+  for (int r = 0; r < kMaxCachedSlots; ++r) hb[r] = uniform64(hb[r]);  // scalar registers, whichever branch ran
   unsigned long long hb_own = 0ull;
-  if (p.hb_in_args) {
+  if (p.rank < kMaxCachedSlots) {
 #pragma unroll
     for (int r = 0; r < kMaxCachedSlots; ++r) hb_own = (r == p.rank) ? hb[r] : hb_own;
-  } else if (p.heap_bases) {
-    hb_own = (unsigned long long)p.heap_bases[p.rank];
+  } else {
+    hb_own = uniform64((unsigned long long)p.heap_bases[p.rank]);
   }
   auto heap_base = [&](int r) -> unsigned long long {
     unsigned long long v = 0;
