@@ -14,7 +14,10 @@ Two timing passes:
     launch's lines out of L2 / last-level cache, the device is synchronised again, and the launch is
     bracketed by GPU events on the launch stream; 25 warm-up and 100 timed launches, mean and median.
 `roofline` prices the flushed launches against the roof that bounds the fused kernel (HBM for the
-slot-sum workloads, MFMA for the others) and also carries the back-to-back per-launch figures;
+slot-sum workloads, MFMA for the others) and also carries the back-to-back per-launch figures and a
+third pass, `launch_ms_flushed_queued`: flushed launches queued behind the flush kernel without a
+synchronisation in between, whose event pairs hold next to nothing of the host's launch path and are
+what a profiler's kernel duration should be compared with;
 `gemm_phase` repeats the measurement with the peers switched off (W = 1), which isolates the MFMA
 phase; `cpu_baseline` times torch's CPU matmul plus the slot reduction on the same workload.
 
@@ -423,17 +426,22 @@ def timed_steps(wl, steps, warmup, graph=False):
 FLUSH_BYTES = int(256e6)
 
 
-def flushed_launches(wl, n_warmup=25, n_repeat=100):
+def flushed_launches(wl, n_warmup=25, n_repeat=100, queued=False):
     """Per-launch GPU-event times in ms under the protocol of the reference's do_bench
     (iris/host/platform/utils.py:137-201): synchronise, zero a 256 MB buffer, synchronise, then the
-    launch alone between two events.  Warm-up launches go through the same sequence."""
+    launch alone between two events.  Warm-up launches go through the same sequence.
+
+    queued=True leaves out the synchronisation between the flush and the launch: the host then queues
+    the events and the launch while the flush kernel still runs, so the event pair holds the kernel and
+    next to nothing of the host's launch path - the figure to compare with a profiler's kernel duration."""
     cache = torch.empty(FLUSH_BYTES // 4, dtype=torch.int, device="cuda")
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
     for i in range(-n_warmup, n_repeat):
         torch.cuda.synchronize()
         cache.zero_()
-        torch.cuda.synchronize()
+        if not queued:
+            torch.cuda.synchronize()
         if i < 0:
             wl.step()
             continue
@@ -447,14 +455,16 @@ def flushed_launches(wl, n_warmup=25, n_repeat=100):
 
 
 def measure(wl, args):
-    """Both timing passes for one prepared workload.  Returns (wall seconds of the K back-to-back
-    steps or None, back-to-back per-launch ms or None, flushed per-launch ms or None)."""
-    wall = b2b = flushed = None
+    """The timing passes for one prepared workload.  Returns (wall seconds of the K back-to-back steps or
+    None, back-to-back per-launch ms or None, flushed per-launch ms or None, the same with the launch
+    queued behind the flush or None)."""
+    wall = b2b = flushed = queued = None
     if args.protocol in ("both", "back_to_back"):
         wall, b2b = timed_steps(wl, args.steps, args.warmup, args.graph)
     if args.protocol in ("both", "flushed"):
         flushed = flushed_launches(wl)
-    return wall, b2b, flushed
+        queued = flushed_launches(wl, n_warmup=5, queued=True)
+    return wall, b2b, flushed, queued
 
 
 def _stats(ms):
@@ -486,7 +496,7 @@ def main():
 
     wl = WORKLOADS[args.workload]()
     wl.setup(iris, args.world)
-    wall, b2b, flushed = measure(wl, args)
+    wall, b2b, flushed, queued = measure(wl, args)
     kernel = _lib.last_kernel() if not isinstance(wl, CopyCalibration) else "torch copy kernel"
     # The roofline prices the flushed launches (the back-to-back ones when only those were run).
     priced = flushed if flushed is not None else b2b
@@ -509,7 +519,8 @@ def main():
                 "unit": unit, "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload, args.world),
                 "kernel": kernel, "flushed": flushed is not None,
                 "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(priced), 5),
-                "launch_ms_flushed": _stats(flushed), "launch_ms_back_to_back": _stats(b2b),
+                "launch_ms_flushed": _stats(flushed), "launch_ms_flushed_queued": _stats(queued),
+                "launch_ms_back_to_back": _stats(b2b),
                 "algorithmic_bytes": bytes_alg, "algorithmic_flops": wl.flops}
 
     out = {
@@ -536,11 +547,12 @@ def main():
         torch.cuda.empty_cache()
         solo = WORKLOADS[args.workload]()
         solo.setup(iris, 1)  # W = 1: same kernel and shape (aux, flags and C still written), no peers to sum
-        wall1, b2b1, flushed1 = measure(solo, args)
+        wall1, b2b1, flushed1, queued1 = measure(solo, args)
         priced1 = flushed1 if flushed1 is not None else b2b1
         t1 = solo.flops / (statistics.mean(priced1) * 1e-3) / 1e12  # per launch, like the roofline
         gp = {"world": 1, "tflops": round(t1, 3), "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4),
               "flushed": flushed1 is not None, "launch_ms_flushed": _stats(flushed1),
+              "launch_ms_flushed_queued": _stats(queued1),
               "launch_ms_back_to_back": _stats(b2b1), "kernel": _lib.last_kernel()}
         if wall1 is not None:
             gp["ms_per_step"] = round(wall1 * 1e3 / args.steps, 5)

@@ -352,12 +352,15 @@ int run_ccl(CclParams p, int distribution, int dtype, void* stream) {
   iris_host::set_last_kernel(name);
   if (p.total_units == 0) return 0;  // this rank owns nothing
 
-  // Launches that move more than the last-level cache holds stream with non-temporal accesses and
-  // four chunks per thread (measured on 8 x 128 MiB: 5.9 instead of 5.1 TB/s); smaller ones keep
-  // cacheable accesses, which is faster when the operands were just produced (6.2 against 4.3 TB/s
-  // for a rank's two-shot share of the same tensors).
+  // Launches that move tens of megabytes stream with non-temporal accesses and four chunks per thread:
+  // their operands are read once, and lines taken into the last-level cache for them would first have to
+  // push out whatever dirty lines it holds (a rank's two-shot share of 8 x 128 MiB after a 256 MB buffer
+  // was zeroed: 74 instead of 92 us; reduce-scatter 42 instead of 62 us; 8 x 128 MiB one-shot 5.9
+  // instead of 5.1 TB/s).  Cacheable accesses win only when the same operands are still cached from a
+  // previous launch (43 against 63 us for the two-shot share), which a collective's inputs - other
+  // ranks' fresh results - are not.  Small launches keep cacheable accesses.
   const long long moved = p.total_units * (long long)(vec * es) * (p.world + (p.mode == CCL_TWO_SHOT ? p.world : 1));
-  const bool stream_nt = vec > 1 && p.mode != CCL_ATOMIC && moved > (512ll << 20);
+  const bool stream_nt = vec > 1 && p.mode != CCL_ATOMIC && moved > (32ll << 20);
   const int upt = stream_nt ? 4 : 2;
   const long long per_wg = (long long)kCclThreads * upt;
   const long long want = (p.total_units + per_wg - 1) / per_wg;
