@@ -32,6 +32,8 @@ def main():
     ap.add_argument("--flush", default="zero", choices=["zero", "read", "none"],
                     help="before every launch: zero a 256 MB buffer (the reference's do_bench), read it, or nothing")
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--deciles", action="store_true",
+                    help="also print, for the last launch, the deciles over workgroups of every phase")
     args = ap.parse_args()
     if not os.path.exists(STAMPS_LIB):
         sys.exit(f"{STAMPS_LIB} is missing: build it with `python -m iris_amd.csrc.build --stamps`")
@@ -99,6 +101,15 @@ def main():
     for name, mean, mx in zip(PHASES, per_phase, per_phase_max):
         print(f"  {name:40s} {statistics.mean(mean):8.2f} | {statistics.mean(mx):8.2f}")
     print(f"  {'first entry -> last stamp':40s} {statistics.mean(spans):8.2f}")
+    if args.deciles:
+        print("last launch, deciles over workgroups (min, 10 %, ..., 90 %, max):")
+        prev = t[:, 0]
+        q = torch.linspace(0, 1, 11, dtype=torch.float64)
+        for i, name in enumerate(PHASES):
+            cur = t[:, i + 1]
+            if float(cur.max()) != 0.0:
+                print(f"  {name:40s} " + " ".join(f"{v:6.2f}" for v in torch.quantile(cur - prev, q).tolist()))
+                prev = cur
 
 
 

@@ -910,37 +910,55 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // last-level cache write back whatever dirty lines it holds to take them in (measured on the
       // 4096 x 4096 x 1376 bf16 launch with seven peers, after a 256 MB buffer had been zeroed: phase 2
       // 68 -> 39 us; with the peers' tiles already cached the two policies tie for the one-shot variant).
-      auto reduce_tile = [&](auto np_tag) {
+      // Chunks are handed to the threads either over the whole kernel tile (RECT false: thread t
+      // takes chunk t of every pass, ownership looked up per chunk) or over one rectangle of it,
+      // rows [r0, r1) and `ncw` chunks from column c0, all of which `rect_owner` reduces (RECT true).
+      auto reduce_chunks = [&](auto np_tag, auto rect_tag, int r0, int r1, int c0, int ncw, int rect_owner) {
         constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
+        constexpr bool RECT = decltype(rect_tag)::value;
         constexpr int NPV = NP > 0 ? NP : 1;
         // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
         // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
         // at a time also with seven peers, and groups below the last row of the matrix are skipped.
         constexpr int G = (NP >= 4 && NW == 8) ? 2 : 4;
         static_assert(PASSES % G == 0, "pass grouping");
-        for (int pg = 0; pg < PASSES; pg += G) {
-          if (m0 + pg * RPP >= p.M) break;
+        const int npasses = RECT ? cdiv((r1 - r0) * ncw, NT) : PASSES;
+        for (int pg = 0; pg < npasses; pg += G) {
+          if (!RECT && m0 + pg * RPP >= p.M) break;
           bool active[G];
           long long eoff[G];
           int owner[G];
           u32x4_t own[G], pv[G][NPV];
 #pragma unroll
           for (int g = 0; g < G; ++g) {
-            const int gm = m0 + (pg + g) * RPP + t_row;
-            owner[g] = p.rank;
-            if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
-              const int t = (gm / p.flag_bm) * ftn + fcol;
-              owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+            int gm, gc, lds_off;
+            if constexpr (RECT) {
+              const unsigned idx = (unsigned)((pg + g) * NT + tid);
+              const unsigned row = idx / (unsigned)ncw;
+              gm = r0 + (int)row;
+              gc = c0 + (int)(idx - row * (unsigned)ncw) * 8;
+              owner[g] = rect_owner;
+              active[g] = gm < r1;
+              lds_off = active[g] ? (gm - m0) * CFG::TROW + (gc - n0) * 2 : 0;
+            } else {
+              gm = m0 + (pg + g) * RPP + t_row;
+              gc = gn;
+              owner[g] = p.rank;
+              if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
+                const int t = (gm / p.flag_bm) * ftn + fcol;
+                owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
+              }
+              active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
+              lds_off = ((pg + g) * RPP + t_row) * CFG::TROW + t_chunk * 16;
             }
-            active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
-            eoff[g] = active[g] ? ((long long)gm * p.s_cm + gn) * 2 : safe_off;
+            eoff[g] = active[g] ? ((long long)gm * p.s_cm + gc) * 2 : safe_off;
             if constexpr (NP > 0) {
 #pragma unroll
               for (int i = 0; i < NP; ++i) {
                 pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
               }
             }
-            own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + (pg + g) * RPP * CFG::TROW);
+            own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(smem + lds_off);
           }
 #pragma unroll
           for (int g = 0; g < G; ++g) {
@@ -984,6 +1002,27 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
             }
           }
         }
+      };
+      // Variants with tile owners (two-shot, reduce-scatter): only the flag tiles this rank owns are
+      // reduced, and a kernel tile may hold none, one or several of them.  When the flag tiles are
+      // large enough to keep the workgroup busy, each owned one is streamed as a rectangle by all
+      // threads, and a kernel tile without an owned flag tile issues nothing at all; with small flag
+      // tiles the threads keep their places in the kernel tile and the stores are predicated.
+      auto reduce_tile = [&](auto np_tag) {
+        const int m1 = min(m0 + BM, p.M), n1 = min(n0 + BN, p.N);
+        const bool by_rect = p.epi != EPI_ONE_SHOT && min(p.flag_bm, BM) * (min(p.flag_bn, BN) / 8) * 2 >= NT;
+        if (!by_rect) {
+          reduce_chunks(np_tag, std::false_type{}, 0, 0, 0, 0, 0);
+          return;
+        }
+        for (int fr = m0 / p.flag_bm; fr * p.flag_bm < m1; ++fr)
+          for (int fc = n0 / p.flag_bn; fc * p.flag_bn < n1; ++fc) {
+            const int owner = owner_of(p.epi, fr * ftn + fc, ftotal, p.world, p.rank);
+            if (!p.all_owners && owner != p.rank) continue;
+            const int r0 = max(m0, fr * p.flag_bm), r1 = min(m1, (fr + 1) * p.flag_bm);
+            const int c0 = max(n0, fc * p.flag_bn), c1 = min(n1, (fc + 1) * p.flag_bn);
+            reduce_chunks(np_tag, std::true_type{}, r0, r1, c0, (c1 - c0) / 8, owner);
+          }
       };
       switch (solo ? -2 : (p.world <= kMaxCachedSlots ? npeers : -1)) {
         case -2: break;  // C was written in phase 1
@@ -1044,8 +1083,11 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   // The two-shot all-reduce does better with one workgroup per tile, handed out by the hardware as CUs
   // free up (measured at W = 8: 16384x4096x1376 322 -> 273 us, 8192x8192x2752 461 -> 417 us,
   // 8192x8192x8192 1059 -> 1009 us); the one-shot variant does worse that way (+3-7 %), launches
-  // without peers do not care.
-  if (p.epi == EPI_TWO_SHOT && p.world > 1 && p.sum_peers) {
+  // without peers do not care.  The same goes for a reduce-scatter whose rank owns one block of
+  // rows: the few tiles that carry the slot sum take half as long again as the others, and a fixed
+  // tile-to-workgroup assignment gives some workgroups two of them.
+  const bool uneven_tiles = p.epi == EPI_TWO_SHOT || (p.epi == EPI_REDUCE_SCATTER && !p.all_owners);
+  if (uneven_tiles && p.world > 1 && p.sum_peers) {
     int per_tile = total;
     if (per_tile % p.num_xcd) per_tile += p.num_xcd - per_tile % p.num_xcd;
     return launch_mfma_grid<CFG, true>(p, device, per_tile, stream);
@@ -1097,6 +1139,15 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
   const int span = cdiv(p.tiles_m * p.tiles_n, p.num_xcd);
   int g = 1;
   while (g * g * 2 <= span && g * 2 <= p.tiles_m) g *= 2;
+  // A reduce-scatter rank sums the slots only for its own band of rows.  With XCD spans that are
+  // close to square that band falls to one or two XCDs, whose CUs then carry all the slow tiles;
+  // taller groups spread it over more XCDs at the price of more operand panels per L2
+  // (8192 x 4096 x 1376, 8 ranks, seven peers: 143 us at height 4, 131 at 8, 114 at 16, 119 at 32).
+  if (p.epi == EPI_REDUCE_SCATTER && !p.all_owners && p.sum_peers && p.world > 1)
+    g = g * 4 < p.tiles_m ? g * 4 : p.tiles_m;
+  // IRIS_HIP_GROUP_M overrides the group height (a tuning aid; results do not depend on the tile order).
+  static const int forced_group_m = [] { const char* e = getenv("IRIS_HIP_GROUP_M"); return e ? atoi(e) : 0; }();
+  if (forced_group_m > 0) g = forced_group_m < p.tiles_m ? forced_group_m : p.tiles_m;
   p.group_m = g;
   static const char* names[3] = {"bf16", "f16", "fp8"};
   char name[96];
