@@ -1142,9 +1142,10 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
   // A reduce-scatter rank sums the slots only for its own band of rows.  With XCD spans that are
   // close to square that band falls to one or two XCDs, whose CUs then carry all the slow tiles;
   // taller groups spread it over more XCDs at the price of more operand panels per L2
-  // (8192 x 4096 x 1376, 8 ranks, seven peers: 143 us at height 4, 131 at 8, 114 at 16, 119 at 32).
+  // (8192 x 4096 x 1376, 8 ranks, seven peers, on one box: 131 us at the default height 8, 114 at
+  // 16, 119 at 32; fetched by the L2s: 207, 290 and 443 MB).
   if (p.epi == EPI_REDUCE_SCATTER && !p.all_owners && p.sum_peers && p.world > 1)
-    g = g * 4 < p.tiles_m ? g * 4 : p.tiles_m;
+    g = g * 2 < p.tiles_m ? g * 2 : p.tiles_m;
   // IRIS_HIP_GROUP_M overrides the group height (a tuning aid; results do not depend on the tile order).
   static const int forced_group_m = [] { const char* e = getenv("IRIS_HIP_GROUP_M"); return e ? atoi(e) : 0; }();
   if (forced_group_m > 0) g = forced_group_m < p.tiles_m ? forced_group_m : p.tiles_m;
