@@ -4,7 +4,7 @@
     python -m iris_amd.bench.phase_stamps [--workload NAME] [--world W] [--flush zero|read|none] [--reps N]
 
 The diagnostic build of the library records the device's constant-rate counter (s_memrealtime) in
-thread 0 of every workgroup at the phase boundaries of its first tile.  This tool runs a workload of
+thread 0 of every workgroup at the phase boundaries of its first eight tiles.  This tool runs a workload of
 bench.py against that build and prints, per phase, the mean and the maximum over the workgroups, and
 the span from the first workgroup's entry to the last workgroup's last store.  Figures include the cost
 of the stamps themselves (one store per phase and workgroup).
@@ -32,8 +32,10 @@ def main():
     ap.add_argument("--flush", default="zero", choices=["zero", "read", "none"],
                     help="before every launch: zero a 256 MB buffer (the reference's do_bench), read it, or nothing")
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--dump", default=None, metavar="FILE.npy",
+                    help="save the last launch's stamps (microseconds, one row of 9 per tile) for other tools")
     ap.add_argument("--deciles", action="store_true",
-                    help="also print, for the last launch, the deciles over workgroups of every phase")
+                    help="also print, for the last launch, the deciles over the stamped tiles of every phase")
     args = ap.parse_args()
     if not os.path.exists(STAMPS_LIB):
         sys.exit(f"{STAMPS_LIB} is missing: build it with `python -m iris_amd.csrc.build --stamps`")
@@ -57,7 +59,7 @@ def main():
 
     wl = bench.WORKLOADS[args.workload or bench.DEFAULT]()
     wl.setup(iris, args.world)
-    max_wgs = 8192
+    max_wgs = 65536  # rows of the stamp buffer: tiles stamped per launch (eight per workgroup at most)
     stamps = torch.zeros((max_wgs, 16), dtype=torch.int64, device="cuda")
     cache = torch.empty(int(256e6) // 4, dtype=torch.int, device="cuda")
     per_phase = [[] for _ in PHASES]
@@ -95,14 +97,18 @@ def main():
             per_phase_max[i].append(float((cur - prev).max()))
             prev = cur
         spans.append(float(t[:, last].max()) - t0)
-    print(f"workload {wl.name}  W={args.world}  kernel {_lib.last_kernel()}  workgroups {t.shape[0]}  flush={args.flush}  "
-          f"{args.reps} launches; microseconds, mean over launches of (mean | max over workgroups)")
+    print(f"workload {wl.name}  W={args.world}  kernel {_lib.last_kernel()}  tiles stamped {t.shape[0]}  flush={args.flush}  "
+          f"{args.reps} launches; microseconds, mean over launches of (mean | max over tiles)")
     print(f"  {'workgroup entry after the first one':40s} {statistics.mean(entry_spread):8.2f}")
     for name, mean, mx in zip(PHASES, per_phase, per_phase_max):
         print(f"  {name:40s} {statistics.mean(mean):8.2f} | {statistics.mean(mx):8.2f}")
     print(f"  {'first entry -> last stamp':40s} {statistics.mean(spans):8.2f}")
+    if args.dump:
+        import numpy
+        os.makedirs(os.path.dirname(os.path.abspath(args.dump)), exist_ok=True)
+        numpy.save(args.dump, (t - t0).numpy())
     if args.deciles:
-        print("last launch, deciles over workgroups (min, 10 %, ..., 90 %, max):")
+        print("last launch, deciles over tiles (min, 10 %, ..., 90 %, max):")
         prev = t[:, 0]
         q = torch.linspace(0, 1, 11, dtype=torch.float64)
         for i, name in enumerate(PHASES):

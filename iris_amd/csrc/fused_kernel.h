@@ -74,14 +74,15 @@ struct FusedParams {
 };
 
 // Diagnostic build (-DIRIS_HIP_PHASE_STAMPS): thread 0 of every workgroup records the constant-rate
-// 100 MHz counter at the phase boundaries of its first tile, into p.stamps[blockIdx.x * 16 + i]:
+// 100 MHz counter at the phase boundaries of its first eight tiles, into row it * gridDim.x + blockIdx.x
+// of p.stamps (16 slots per row, slot i):
 //   0 kernel entry, 1 first operands in LDS, 2 K loop done, 3 tile staged in LDS, 4 phase-1 stores
 //   issued, 5 phase-1 stores acknowledged, 6 own flags raised and peers' flags seen, 7 phase-2 stores
 //   issued, 8 last store acknowledged.  The regular build compiles the macro away.
 #ifdef IRIS_HIP_PHASE_STAMPS
 #define PHASE_STAMP(i)                                                                         \
   do {                                                                                         \
-    if (p.stamps && threadIdx.x == 0 && it == 0) p.stamps[blockIdx.x * 16 + (i)] = wall_clock64(); \
+    if (p.stamps && threadIdx.x == 0 && it < 8) p.stamps[(it * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64(); \
   } while (0)
 #else
 #define PHASE_STAMP(i) \
