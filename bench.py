@@ -8,7 +8,8 @@ sit in HBM (peers' partial results and flags staged before the timed region).
 
 Two timing passes:
   * back to back: W untimed steps, then K timed steps between two device synchronisations; `value` is
-    the whole-job throughput of those K steps in TFLOP/s (2*M*N*K flop per step, wall clock).
+    the whole-job throughput of those K steps in TFLOP/s (2*M*N*K flop per step, wall clock).  K more
+    steps follow with a GPU event pair around every launch (`launch_ms_back_to_back`).
   * flushed, the protocol of the reference's iris.do_bench (iris/host/platform/utils.py:137-201):
     before every launch the device is synchronised, a 256 MB buffer is zeroed to push the previous
     launch's lines out of L2 / last-level cache, the device is synchronised again, and the launch is
@@ -384,8 +385,8 @@ def measured_traffic(workload, world):
 
 
 def timed_steps(wl, steps, warmup, graph=False):
-    """W untimed steps, then K timed ones between device synchronisations; every timed launch is also
-    bracketed by GPU events on the launch stream.  With graph=True the K steps are captured into one
+    """W untimed steps, then K timed ones between device synchronisations (the wall-clock figure), then K
+    more with every launch bracketed by GPU events on the launch stream (the per-launch figures).  With graph=True the K steps are captured into one
     HIP graph after the warm-up and the timed region is one replay of it (no host work between the
     launches; the per-launch time is then the replay time divided by K)."""
     for _ in range(warmup):
@@ -409,15 +410,22 @@ def timed_steps(wl, steps, warmup, graph=False):
         wall = time.perf_counter() - t0
         wl.ctx.check_status()
         return wall, [start.elapsed_time(end) / steps] * steps
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    wl.ctx.check_status()
+    # The per-launch figures come from a second run of K steps: an event pair around every launch puts
+    # two more packets per step on the queue (about 5 us of gaps per step), which the timed region above
+    # should not pay for.
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
         wl.step()
         ends[i].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     wl.ctx.check_status()
     per_launch_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
     return wall, per_launch_ms

@@ -341,8 +341,8 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
       const float* part = (const float*)(smem + CFG::OPERANDS + w * CFG::WAVE_BYTES) + row * CFG::RED_STRIDE + 4 * c;
       s4 += *(const LDS_AS f32x4_t*)(LDS_AS const char*)((const char*)part);
     }
-    own.x = (unsigned)Out::from_float(s4.x * p.scale) | ((unsigned)Out::from_float(s4.y * p.scale) << 16);
-    own.y = (unsigned)Out::from_float(s4.z * p.scale) | ((unsigned)Out::from_float(s4.w * p.scale) << 16);
+    own.x = Out::pack(s4.x * p.scale, s4.y * p.scale);
+    own.y = Out::pack(s4.z * p.scale, s4.w * p.scale);
   }
   const unsigned long long c_own = (unsigned long long)p.C;
   int owner = p.rank;
@@ -391,7 +391,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
     u32x2_t res;
 #pragma unroll
     for (int e = 0; e < 2; ++e)
-      res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
+      res[e] = Out::pack(sum[2 * e], sum[2 * e + 1]);
     store_result(res);
   };
 

@@ -27,15 +27,31 @@ __device__ __forceinline__ float f16_bits_to_float(unsigned short b) {
   return (float)__builtin_bit_cast(_Float16, b);
 }
 
+// Two floats rounded (to nearest even) and packed into one word, `lo` in the low half: one
+// v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 instead of two conversions and a merge.
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+__device__ __forceinline__ unsigned pack_f16(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, half2_t));
+}
+
 // Output element kinds of the 16-bit epilogue.
 struct OutBF16 {
   static __device__ __forceinline__ float to_float(unsigned short b) { return bf16_bits_to_float(b); }
   static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_bf16_bits(f); }
+  static __device__ __forceinline__ unsigned pack(float lo, float hi) { return pack_bf16(lo, hi); }
   static constexpr bool kFp32SumInReference = false;
 };
 struct OutF16 {
   static __device__ __forceinline__ float to_float(unsigned short b) { return f16_bits_to_float(b); }
   static __device__ __forceinline__ unsigned short from_float(float f) { return float_to_f16_bits(f); }
+  static __device__ __forceinline__ unsigned pack(float lo, float hi) { return pack_f16(lo, hi); }
   static constexpr bool kFp32SumInReference = true;
 };
 

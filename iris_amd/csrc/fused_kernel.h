@@ -803,13 +803,12 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            unsigned short h[4];
+            float h[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              h[e] = Out::from_float(acc_read(acc.v[mb][nb][4 * q + e]) * p.scale + badd[mb]);
+            for (int e = 0; e < 4; ++e) h[e] = acc_read(acc.v[mb][nb][4 * q + e]) * p.scale + badd[mb];
             u32x2_t w;
-            w.x = (unsigned)h[0] | ((unsigned)h[1] << 16);
-            w.y = (unsigned)h[2] | ((unsigned)h[3] << 16);
+            w.x = Out::pack(h[0], h[1]);
+            w.y = Out::pack(h[2], h[3]);
             const int trow = wm * TM + mb * 32 + acc_col(lane);
             const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
             *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
@@ -990,7 +989,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
             u32x4_t res;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              res[e] = (unsigned)Out::from_float(sum[2 * e]) | ((unsigned)Out::from_float(sum[2 * e + 1]) << 16);
+              res[e] = Out::pack(sum[2 * e], sum[2 * e + 1]);
             if (active[g]) {
               if (p.epi == EPI_TWO_SHOT) {
                 __builtin_nontemporal_store(res, (u32x4_t*)(c_own + eoff[g]));
