@@ -166,6 +166,37 @@ __device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, in
   }
 }
 
+// One look at the peers' flags that wait_peer_flags would wait for, without waiting: true when
+// every flag this thread looked at was already 1, in which case the thread has also passed an
+// acquire fence at system scope.  A workgroup barrier must follow before anybody reads the peers' data.
+template <int KM, int KN, int NT>
+__device__ __forceinline__ bool probe_peer_flags(const FusedParams& p, int m0, int n0, int tid) {
+  const int m1 = min(m0 + KM, p.M), n1 = min(n0 + KN, p.N);
+  const int ftn = cdiv(p.N, p.flag_bn);
+  const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
+  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
+  const int nfn = fn_hi - fn_lo + 1;
+  const int nft = (fm_hi - fm_lo + 1) * nfn;
+  const int items = nft * p.world;
+  bool up = true, looked = false;
+  for (int i = tid; i < items; i += NT) {
+    const int r = i % p.world;
+    const int f = i / p.world;
+    if (r == p.rank) continue;
+    const int t = (fm_lo + f / nfn) * ftn + fn_lo + f % nfn;
+    if (!p.all_owners && owner_of(p.epi, t, ftotal, p.world, p.rank) != p.rank) continue;
+    const int* flag = (const int*)slot_ptr(p.heap_bases, p.locks + t, p.rank, r);
+    up = up && (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 1);
+    looked = true;
+  }
+  // Only the threads that looked at a flag invalidate the caches (as only the polling threads do in
+  // wait_peer_flags): the caches are the compute unit's, and an invalidation per wave of every
+  // workgroup costs more than the probe saves.
+  if (looked && up) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+  return up;
+}
+
 // ------------------------------------------------------------------------------------------------
 // MFMA kernel configuration
 // ------------------------------------------------------------------------------------------------
@@ -879,13 +910,19 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // (no L2 write-back is needed any more).  Likewise the peers' flags are polled (system-scope
       // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
       // every wave poll and run ahead measured slower.
+      // The peers' flags are looked at once while the own stores are still on their way: when all of
+      // them are up already - peers that finished first - their round trip hides behind that wait
+      // and the polling after the own flags are raised is skipped.
+      const bool up_already = solo ? true : probe_peer_flags<BM, BN, NT>(p, m0, n0, tid);
       wait_vmcnt<0>();
-      __syncthreads();
+      const bool all_up = __syncthreads_and(up_already);
       PHASE_STAMP(5);
       raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
       if (!solo) {
-        wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
-        __syncthreads();
+        if (!all_up) {
+          wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
+          __syncthreads();
+        }
       }
       PHASE_STAMP(6);
 
