@@ -441,6 +441,36 @@ def test_unstaged_peer_flags_time_out():
     assert torch.all(ws.locks.cpu() == 1), "own flags are raised before waiting"
 
 
+@pytest.mark.parametrize("M,N,K,variant", [(512, 384, 96, "one_shot"), (512, 384, 96, "two_shot"),
+                                           (32, 1168, 1360, "one_shot"), (3072, 3072, 80, "one_shot")])
+def test_unregistered_context_tensor_gives_the_same_bits(M, N, K, variant):
+    """The kernels take the heap bases as kernel arguments when the host has registered the context
+    tensor's contents, and load them from the tensor otherwise (a binding that never registers).
+    Both routes must produce the same aux, flags and C; the sizes cover the 128x128, 32x32 (decode)
+    and 256x256 kernels."""
+    W, rank, dtype = 4, 1, torch.bfloat16
+    A, B = randint_cpu((M, K), 20, dtype), randint_cpu((K, N), 21, dtype)
+    peers = [randn_cpu((M, N), 200 + r, dtype) for r in range(W)]
+    fbm = 32 if M == 32 else 128
+    cfg = iris.FusedConfig(block_size_m=fbm, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, fbm, 64, variant, "fp32")
+    kernels = []
+    for registered in (True, False):
+        ctx = _ctx(W, rank)
+        if not registered:
+            ctx._forget_device_context()
+        assert ctx._context_registered == registered
+        dC, ws, kernel = _run_all_reduce(ctx, A, B, peers, cfg)
+        kernels.append(kernel)
+        assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"aux, registered={registered}")
+        assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+        got = slot_copies(ctx, dC)
+        for r in range(W if variant == "two_shot" else 1):
+            slot = r if variant == "two_shot" else rank
+            assert_bits_equal(got[slot], exp["C"][slot], f"{kernel} C in slot {slot}, registered={registered}")
+    assert kernels[0] == kernels[1] and kernels[0].startswith("mfma_")
+
+
 def test_heap_tensors_outlive_their_context(monkeypatch):
     """The heap allocation is released with its last tensor, not with the context object."""
     from iris_amd.host import hip as hip_mod

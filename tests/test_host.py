@@ -306,6 +306,27 @@ def test_null_context_tensor_is_rejected_before_any_launch():
         assert rc == 1 and "context_tensor" in _lib.last_error()
 
 
+def test_context_registration_checks_its_arguments():
+    """Registering what a context tensor holds touches no device memory: the host copy is read, the
+    device pointer only remembered.  Bad contents are argument errors; unregistering an unknown
+    pointer is not."""
+    lib = _lib.library()
+    words = (ctypes.c_int64 * 27)(3, 8, *[0x7000_0000_0000 + (r << 30) for r in range(8)])
+    host, dev, null = ctypes.cast(words, ctypes.c_void_p), ctypes.c_void_p(0x20000), ctypes.c_void_p(0)
+    assert lib.iris_hip_register_context(dev, host, 27) == 0 and _lib.last_error() == ""
+    assert lib.iris_hip_register_context(dev, host, 27) == 0        # again: replaces the entry
+    assert lib.iris_hip_register_context(null, host, 27) == 1 and "must not be NULL" in _lib.last_error()
+    assert lib.iris_hip_register_context(dev, null, 27) == 1 and "must not be NULL" in _lib.last_error()
+    assert lib.iris_hip_register_context(dev, host, 2) == 1 and "at least 3 words" in _lib.last_error()
+    assert lib.iris_hip_register_context(dev, host, 9) == 1 and "bad context contents" in _lib.last_error()  # 8 bases need 10 words
+    bad_rank = (ctypes.c_int64 * 10)(8, 8, *([0] * 8))
+    assert lib.iris_hip_register_context(dev, ctypes.cast(bad_rank, ctypes.c_void_p), 10) == 1
+    assert "bad context contents" in _lib.last_error()
+    assert lib.iris_hip_unregister_context(dev) == 0
+    assert lib.iris_hip_unregister_context(dev) == 0                # unknown by now: still fine
+    assert lib.iris_hip_unregister_context(null) == 0
+
+
 def test_device_span_releases_its_memory_exactly_once():
     """The object torch keeps alive for the heap's tensors owns the allocation."""
     from iris_amd.host.heap import _DeviceSpan
