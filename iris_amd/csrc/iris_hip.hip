@@ -432,6 +432,19 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   else if (p.M <= 32 && epi_has_flags(p.epi) && p.gather == GATHER_NONE && p.world <= 8 && !p.bias) kind = TILE_DECODE;
   else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
+  // IRIS_HIP_TILE = big | small | small2 | skinny overrides the choice among the tiled kernels (a tuning
+  // aid; results do not depend on the tile shape beyond the order of the fp32 sums over K).
+  static const int forced_tile = [] {
+    const char* e = getenv("IRIS_HIP_TILE");
+    if (!e) return -1;
+    if (!strcmp(e, "big")) return (int)TILE_BIG;
+    if (!strcmp(e, "small")) return (int)TILE_SMALL;
+    if (!strcmp(e, "small2")) return (int)TILE_SMALL2;
+    if (!strcmp(e, "skinny")) return (int)TILE_SKINNY;
+    return -1;
+  }();
+  if (forced_tile >= 0 && kind != TILE_DECODE && !(forced_tile == TILE_SKINNY && p.gather == GATHER_M && p.M_local % 64))
+    kind = forced_tile;
   const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
