@@ -866,6 +866,27 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       const int ftn1 = cdiv(p.N, p.flag_bn);
       const int ftotal1 = cdiv(p.M, p.flag_bm) * ftn1;
       const unsigned long long c_base = (unsigned long long)p.C;
+      if (p.epi == EPI_ATOMIC) {
+        // The tile is added into every rank's C (iris/mem/triton/context.py:689-702) with packed 16-bit
+        // atomics of one dword each.  Dword d of a pass belongs to thread d mod NT, so that one wave
+        // instruction covers 256 contiguous bytes (two whole lines for the L2's atomic units); with
+        // each thread adding the four dwords of its own 16-byte chunk an instruction touched eight
+        // lines with eight dwords each, and the launch ran at a quarter of the rate.
+        constexpr int DPR = BN / 2;                   // dwords per tile row
+        constexpr int DPP = RPP * DPR;                // dwords per pass (= 4 * NT)
+        for (int ps = 0; ps < PASSES; ++ps) {
+#pragma unroll
+          for (int j = 0; j < DPP / NT; ++j) {
+            const int d = j * NT + tid;
+            const int row = ps * RPP + d / DPR, dc = d % DPR;
+            const int gm = m0 + row, gc = n0 + 2 * dc;
+            if (gm >= p.M || gc >= p.N) continue;
+            const unsigned w = *(const LDS_AS unsigned*)(LDS_AS char*)(smem + row * CFG::TROW + dc * 4);
+            const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gc) * 2;
+            for (int pr = 0; pr < p.world; ++pr) atomic_add_packed<Out>((char*)(in_slot(c_base, pr) + eoff), w);
+          }
+        }
+      } else
 #pragma unroll 4
       for (int ps = 0; ps < PASSES; ++ps) {
         const int gm = m0 + ps * RPP + t_row;
@@ -875,13 +896,6 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           if (p.epi == EPI_ALL_GATHER) {
             // the tile goes to every rank's gathered output (iris/mem/triton/context.py:841-864)
             for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
-          } else if (p.epi == EPI_ATOMIC) {
-            // the tile is added into every rank's C (iris/mem/triton/context.py:689-702)
-            for (int pr = 0; pr < p.world; ++pr) {
-              char* dst = (char*)(in_slot(c_base, pr) + eoff);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) atomic_add_packed<Out>(dst + 4 * e, v[e]);
-            }
           } else if (flags) {
             store16_system(out1 + eoff, v);  // aux: read by the peers as soon as the flag is up
           } else {

@@ -91,6 +91,28 @@ struct Chunk<E, 1> {
 };
 
 template <class E>
+struct Chunk<E, 2> {  // two 16-bit elements: the unit of the packed atomics
+  float v[2];
+  template <bool NT> __device__ __forceinline__ void load(const char* p) {
+    const unsigned w = *(const unsigned*)p;
+    unsigned short lo = (unsigned short)(w & 0xFFFFu), hi = (unsigned short)(w >> 16);
+    v[0] = E::load((const char*)&lo);
+    v[1] = E::load((const char*)&hi);
+  }
+  __device__ __forceinline__ unsigned pack() const {
+    unsigned short lo, hi;
+    E::store((char*)&lo, v[0]);
+    E::store((char*)&hi, v[1]);
+    return (unsigned)lo | ((unsigned)hi << 16);
+  }
+  template <bool NT> __device__ __forceinline__ void store(char* p) const { *(unsigned*)p = pack(); }
+  __device__ __forceinline__ void atomic_add_to(char* p) const {
+    using Out = typename std::conditional<E::kFp32SumInReference, OutF16, OutBF16>::type;
+    atomic_add_packed<Out>(p, pack());
+  }
+};
+
+template <class E>
 struct Chunk<E, 8> {  // eight 16-bit elements
   float v[8];
   template <bool NT> __device__ __forceinline__ void load(const char* p) {
@@ -307,7 +329,12 @@ int run_ccl(CclParams p, int distribution, int dtype, void* stream) {
   bool vec_ok = p.s_in == 1 && p.s_on == 1 && aligned16(p.in) && aligned16(p.out) &&
                 (p.s_im * es) % 16 == 0 && (p.s_om * es) % 16 == 0 && p.N % vec_full == 0;
   if (tiled && p.bn % vec_full) vec_ok = false;
-  const int vec = vec_ok ? vec_full : 1;
+  int vec = vec_ok ? vec_full : 1;
+  // The atomic variant adds one dword at a time (packed 16-bit pairs, or one float): with a dword per
+  // thread a wave instruction covers 256 contiguous bytes, two whole lines for the L2's atomic units;
+  // with a 16-byte chunk per thread it touched eight lines with eight dwords each and the launch ran
+  // at a third of the rate.
+  if (p.mode == CCL_ATOMIC && vec_ok) vec = es == 4 ? 1 : 2;
 
   if (tiled) {
     p.tiles_m = cdiv(p.M, p.bm);
@@ -372,7 +399,11 @@ int run_ccl(CclParams p, int distribution, int dtype, void* stream) {
     if (stream_nt) launch_for_world<E, V, 4, true>(p, grid, s); \
     else launch_for_world<E, V, 2, false>(p, grid, s);          \
   } while (0)
-  if (dtype == IRIS_HIP_BF16) { if (vec == 8) CCL_LAUNCH(ElemBF16, 8); else CCL_LAUNCH(ElemBF16, 1); }
+  if (vec == 2) {  // atomic variant only
+    if (dtype == IRIS_HIP_BF16) launch_for_world<ElemBF16, 2, 2, false>(p, grid, s);
+    else launch_for_world<ElemF16, 2, 2, false>(p, grid, s);
+  }
+  else if (dtype == IRIS_HIP_BF16) { if (vec == 8) CCL_LAUNCH(ElemBF16, 8); else CCL_LAUNCH(ElemBF16, 1); }
   else if (dtype == IRIS_HIP_FP16) { if (vec == 8) CCL_LAUNCH(ElemF16, 8); else CCL_LAUNCH(ElemF16, 1); }
   else { if (vec == 4) CCL_LAUNCH(ElemF32, 4); else CCL_LAUNCH(ElemF32, 1); }
 #undef CCL_LAUNCH

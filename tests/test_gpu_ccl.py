@@ -44,7 +44,10 @@ def test_all_reduce_matches_oracle(variant, M, N, bm, bn, dtype):
         cfg.all_reduce_distribution = 0  # as the reference test does
     ws = ctx.ccl.all_reduce_preamble(d_out, d_in, config=cfg)
     ctx.ccl.all_reduce(d_out, d_in, config=cfg, workspace=ws)
-    assert "vec" in _lib.last_kernel() and "vec1" not in _lib.last_kernel()
+    if variant == "atomic":  # one dword per thread: packed pairs of 16-bit values, or one float
+        assert _lib.last_kernel().endswith("vec1" if dtype == torch.float32 else "vec2"), _lib.last_kernel()
+    else:
+        assert "vec" in _lib.last_kernel() and "vec1" not in _lib.last_kernel()
     exp = oracle.ccl_all_reduce(inputs, [torch.zeros((M, N), dtype=dtype)] * W, rank, variant, bm, bn,
                                 cfg.swizzle_size, cfg.comm_sms, cfg.all_reduce_distribution)
     got = slot_copies(ctx, d_out)
