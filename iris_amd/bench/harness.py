@@ -8,6 +8,7 @@ command line :399-520) of the reference.
 import argparse
 import csv
 import io
+import gc
 import itertools
 import json
 import re
@@ -277,35 +278,47 @@ def _run_world(benchmarks, world_size, rank, overrides, skips, heap_size, n_warm
         declares_ranks = any(ax.name == RANKS_AXIS for ax in bdef.axes)
         if world_size not in _world_sizes(bdef, overrides, skips):
             continue
-        # A fresh heap per benchmark: the bump allocator never frees, and a sweep allocates per combination.
-        ctx = make_context(heap_size, world_size, rank)
         axes = [AxisDef(ax.name, _values(ax, overrides, skips)) for ax in bdef.axes if ax.name != RANKS_AXIS]
         if any(not ax.values for ax in axes):
             continue  # an axis emptied by --skip_* drops the whole benchmark
-        for combo in itertools.product(*[ax.values for ax in axes]):
-            params = {RANKS_AXIS: world_size} if (declares_ranks or RANKS_AXIS in overrides) else {}
-            params.update(zip([ax.name for ax in axes], combo))
-            state = State(params, n_warmup, n_repeat)
-            try:
-                bdef.fn(state, ctx)
-            except _Skip as skip:
-                results.append(Result(bdef.name, params, 0.0, [], skipped=True, skip_reason=skip.reason,
-                                      world_size=world_size))
-                continue
-            if state._exec_fn is None:
-                raise RuntimeError(f"Benchmark '{bdef.name}' with params {params} did not call state.exec(fn). "
-                                   f"Every benchmark must register a callable to time.")
-            times = time_fn(state._exec_fn, barrier_fn=ctx.barrier, preamble_fn=state._preamble_fn,
-                            n_warmup=state._n_warmup, n_repeat=state._n_repeat, return_mode="all")
-            mean_ms = statistics.mean(times)
-            per_second = (lambda n: n / (mean_ms * 1e-3)) if mean_ms > 0 else (lambda n: None)
-            results.append(Result(
-                bdef.name, params, mean_ms, times,
-                bandwidth_gbps=None if state._bytes is None else per_second(state._bytes / 1e9),
-                tflops=None if state._flops is None else per_second(state._flops / 1e12),
-                counters=dict(state._counters), world_size=world_size))
+        # A fresh heap per benchmark: the bump allocator never frees, and a sweep allocates per combination.
+        ctx = make_context(heap_size, world_size, rank)
+        results += _run_benchmark(bdef, axes, ctx, world_size, declares_ranks or RANKS_AXIS in overrides,
+                                  n_warmup, n_repeat, time_fn)
         ctx.barrier()
+        # The heap lives as long as its last tensor: everything the benchmark allocated (tensors held by
+        # the callables it registered included) went out of scope with _run_benchmark; collect what sits
+        # in reference cycles before the next benchmark asks for a heap of its own.
         del ctx
+        gc.collect()
+    return results
+
+
+def _run_benchmark(bdef, axes, ctx, world_size, show_ranks, n_warmup, n_repeat, time_fn):
+    """All parameter combinations of one benchmark on one context."""
+    results = []
+    for combo in itertools.product(*[ax.values for ax in axes]):
+        params = {RANKS_AXIS: world_size} if show_ranks else {}
+        params.update(zip([ax.name for ax in axes], combo))
+        state = State(params, n_warmup, n_repeat)
+        try:
+            bdef.fn(state, ctx)
+        except _Skip as skip:
+            results.append(Result(bdef.name, params, 0.0, [], skipped=True, skip_reason=skip.reason,
+                                  world_size=world_size))
+            continue
+        if state._exec_fn is None:
+            raise RuntimeError(f"Benchmark '{bdef.name}' with params {params} did not call state.exec(fn). "
+                               f"Every benchmark must register a callable to time.")
+        times = time_fn(state._exec_fn, barrier_fn=ctx.barrier, preamble_fn=state._preamble_fn,
+                        n_warmup=state._n_warmup, n_repeat=state._n_repeat, return_mode="all")
+        mean_ms = statistics.mean(times)
+        per_second = (lambda n: n / (mean_ms * 1e-3)) if mean_ms > 0 else (lambda n: None)
+        results.append(Result(
+            bdef.name, params, mean_ms, times,
+            bandwidth_gbps=None if state._bytes is None else per_second(state._bytes / 1e9),
+            tflops=None if state._flops is None else per_second(state._flops / 1e12),
+            counters=dict(state._counters), world_size=world_size))
     return results
 
 

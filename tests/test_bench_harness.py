@@ -161,3 +161,34 @@ def test_range_helpers_and_registration():
     assert len(harness._registry) == before + 1
     assert [ax.name for ax in harness._registry[-1].axes] == ["a", "b"]  # declaration order = sweep order
     harness._registry.pop()
+
+
+def test_a_benchmarks_tensors_are_gone_before_the_next_context_is_made():
+    """Every benchmark gets a heap of its own, and a heap lives as long as its last tensor: what one
+    benchmark allocated - also what the callables it registered hold on to - must be released before
+    the next benchmark's context is created, or the heaps pile up (3 x 128 GiB does not fit a GPU)."""
+    import weakref
+
+    import iris_amd as iris
+
+    allocated, alive_at_creation = [], []
+
+    def make_context(heap_size, world_size, rank):
+        alive_at_creation.append(sum(ref() is not None for ref in allocated))
+        return iris.iris(1 << 20, num_ranks=world_size, rank=rank, device="cpu")
+
+    def make_benchmark(name):
+        @bench.axis("num_ranks", [2])
+        @bench.axis("M", [64, 128])
+        def fn(state, ctx):
+            x = ctx.zeros((state["M"], 32), dtype=torch.float32)
+            y = ctx.zeros((state["M"], 32), dtype=torch.float32)
+            allocated.extend([weakref.ref(x), weakref.ref(y)])
+            state.exec(lambda: y.copy_(x), preamble_fn=y.zero_)
+        return harness.BenchmarkDef(name, fn, fn._bench_axes)
+
+    results = harness.run_registered([make_benchmark("first"), make_benchmark("second"), make_benchmark("third")],
+                                     make_context=make_context, time_fn=fake_timer, n_warmup=1, n_repeat=2)
+    assert len(results) == 6
+    assert alive_at_creation == [0, 0, 0]
+    assert all(ref() is None for ref in allocated)
