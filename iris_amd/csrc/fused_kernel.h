@@ -895,21 +895,21 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gn) * 2;
           if (p.epi == EPI_ALL_GATHER) {
             // the tile goes to every rank's gathered output (iris/mem/triton/context.py:841-864)
-            for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
+            for (int pr = 0; pr < p.world; ++pr) __builtin_nontemporal_store(v, (u32x4_t*)(in_slot(c_base, pr) + eoff));
           } else if (flags) {
             store16_system(out1 + eoff, v);  // aux: read by the peers as soon as the flag is up
           } else {
-            *(u32x4_t*)(out1 + eoff) = v;
+            __builtin_nontemporal_store(v, (u32x4_t*)(out1 + eoff));
           }
           if (solo) {
             int owner = p.rank;
             if (p.epi != EPI_ONE_SHOT) owner = owner_of(p.epi, (gm / p.flag_bm) * ftn1 + gn / p.flag_bn, ftotal1, p.world, p.rank);
             if (p.all_owners || owner == p.rank) {
               if (p.epi == EPI_TWO_SHOT) {
-                for (int pr = 0; pr < p.world; ++pr) *(u32x4_t*)(in_slot(c_base, pr) + eoff) = v;
+                for (int pr = 0; pr < p.world; ++pr) __builtin_nontemporal_store(v, (u32x4_t*)(in_slot(c_base, pr) + eoff));
               } else {
                 const int dst = p.all_owners ? owner : p.rank;
-                *(u32x4_t*)(in_slot(c_base, dst) + eoff) = v;
+                __builtin_nontemporal_store(v, (u32x4_t*)(in_slot(c_base, dst) + eoff));
               }
             }
           }
