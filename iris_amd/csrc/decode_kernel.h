@@ -189,6 +189,9 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
       }
     }
     if (lane == 0) *(LDS_AS int*)(LDS_AS char*)(smem + CFG::WORD_AREA) = early ? 1 : 0;
+    // The helper has nothing else to do: it waits here for the peers' tiles, so that behind the barrier
+    // that ends the K phase they are known to be in LDS.
+    wait_vmcnt<0>();
   }
 
   // ---- operand loaders ---------------------------------------------------------------------------
@@ -398,21 +401,21 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   if (valid) store8_system(p.aux + eoff, own);  // read by the peers as soon as the flag is up
   if (solo && reduces) store_result(own);
   PHASE_STAMP(4);
-  // Publish (as in the tiled kernel): stores acknowledged, workgroup barrier, flags.  The helper wave's
-  // wait is for the peers' tiles it asked for, so behind the barrier the slot sum has everything it needs
-  // and does not stand between the aux stores and the flags.
+  // When the helper found every flag up, the peers' tiles are in LDS by now (it waited for them before
+  // the barrier above): the slot sum and the C stores go out right behind the aux stores, and one wait
+  // covers both before the flags are raised - one memory round trip less in the chain.
+  const bool have_peers = !solo && nft <= 64 && p.hb_in_args && *(const LDS_AS int*)(LDS_AS char*)(smem + CFG::WORD_AREA) != 0;
+  if (have_peers && reduces) reduce_and_store(true);
+  // Publish (as in the tiled kernel): stores acknowledged, workgroup barrier, flags.
   wait_vmcnt<0>();
   __syncthreads();
   PHASE_STAMP(5);
-  const bool have_peers = !solo && nft <= 64 && p.hb_in_args && *(const LDS_AS int*)(LDS_AS char*)(smem + CFG::WORD_AREA) != 0;
   raise_flags<CFG::BM, CFG::BN, CFG::NT, true>(p, 0, n0, tid);
-  if (solo) return;
-  if (!have_peers) {
-    wait_peer_flags<CFG::BM, CFG::BN, CFG::NT>(p, 0, n0, tid);
-    __syncthreads();
-  }
+  if (solo || have_peers) return;
+  wait_peer_flags<CFG::BM, CFG::BN, CFG::NT>(p, 0, n0, tid);
+  __syncthreads();
   PHASE_STAMP(6);
-  if (reduces) reduce_and_store(have_peers);
+  if (reduces) reduce_and_store(false);
   PHASE_STAMP(7);
 }
 
