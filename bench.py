@@ -14,11 +14,13 @@ Two timing passes:
     before every launch the device is synchronised, a 256 MB buffer is zeroed to push the previous
     launch's lines out of L2 / last-level cache, the device is synchronised again, and the launch is
     bracketed by GPU events on the launch stream; 25 warm-up and 100 timed launches, mean and median.
-`roofline` prices the flushed launches against the roof that bounds the fused kernel (HBM for the
-slot-sum workloads, MFMA for the others) and also carries the back-to-back per-launch figures and a
-third pass, `launch_ms_flushed_queued`: flushed launches queued behind the flush kernel without a
-synchronisation in between, whose event pairs hold next to nothing of the host's launch path and are
-what a profiler's kernel duration should be compared with;
+A third pass, `launch_ms_flushed_queued`, repeats the flushed launches without the synchronisation
+between flush and launch: the launch is queued while the flush kernel still runs, so its event pair
+holds the kernel and next to nothing of the host's launch path (5-8 us through Python, ctypes and the
+HIP runtime on an idle queue) and agrees with a profiler's kernel duration for the same command.
+`roofline` prices those launches (`priced_on`) against the roof that bounds the fused kernel (HBM for
+the slot-sum workloads, MFMA for the others); `frac_do_bench` is the same fraction priced on the literal
+do_bench launches, host path included; the back-to-back per-launch figures are carried as well;
 `gemm_phase` repeats the measurement with the peers switched off (W = 1), which isolates the MFMA
 phase; `cpu_baseline` times torch's CPU matmul plus the slot reduction on the same workload.
 
@@ -506,8 +508,13 @@ def main():
     wl.setup(iris, args.world)
     wall, b2b, flushed, queued = measure(wl, args)
     kernel = _lib.last_kernel() if not isinstance(wl, CopyCalibration) else "torch copy kernel"
-    # The roofline prices the flushed launches (the back-to-back ones when only those were run).
-    priced = flushed if flushed is not None else b2b
+    # The roofline prices the kernel's duration after a cache flush: the flushed launches whose event
+    # pairs hold the kernel alone (queued behind the flush), which is what a profiler's kernel average
+    # of the same command reads.  The literal do_bench sequence (a host synchronisation between flush
+    # and launch, so that the pair also holds the host's launch path) is reported beside it as
+    # launch_ms_flushed / frac_do_bench.  Back-to-back launches are priced when only those were run.
+    priced = queued if queued is not None else (flushed if flushed is not None else b2b)
+    priced_on = "launch_ms_flushed_queued" if queued is not None else ("launch_ms_flushed" if flushed is not None else "launch_ms_back_to_back")
     launch_ms = statistics.mean(priced)
     if wall is not None:
         ms_per_step = wall * 1e3 / args.steps
@@ -523,9 +530,11 @@ def main():
     else:
         peak, unit = PEAK[wl.dtype]
         achieved = wl.flops / (launch_ms * 1e-3) / 1e12
+    per_ms = bytes_alg / 1e6 if wl.bound == "hbm" else wl.flops / 1e9  # achieved = per_ms / launch_ms, in GB/s or TFLOP/s
     roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "achieved": round(achieved, 2), "peak": peak,
                 "unit": unit, "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload, args.world),
-                "kernel": kernel, "flushed": flushed is not None,
+                "kernel": kernel, "flushed": flushed is not None, "priced_on": priced_on,
+                "frac_do_bench": round(per_ms / statistics.mean(flushed) / peak, 4) if flushed is not None else None,
                 "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(priced), 5),
                 "launch_ms_flushed": _stats(flushed), "launch_ms_flushed_queued": _stats(queued),
                 "launch_ms_back_to_back": _stats(b2b),
@@ -556,9 +565,11 @@ def main():
         solo = WORKLOADS[args.workload]()
         solo.setup(iris, 1)  # W = 1: same kernel and shape (aux, flags and C still written), no peers to sum
         wall1, b2b1, flushed1, queued1 = measure(solo, args)
-        priced1 = flushed1 if flushed1 is not None else b2b1
+        priced1 = queued1 if queued1 is not None else (flushed1 if flushed1 is not None else b2b1)
         t1 = solo.flops / (statistics.mean(priced1) * 1e-3) / 1e12  # per launch, like the roofline
         gp = {"world": 1, "tflops": round(t1, 3), "frac_of_mfma_peak": round(t1 / PEAK[solo.dtype][0], 4),
+              "frac_of_mfma_peak_do_bench": (round(solo.flops / (statistics.mean(flushed1) * 1e-3) / 1e12 / PEAK[solo.dtype][0], 4)
+                                             if flushed1 is not None else None),
               "flushed": flushed1 is not None, "launch_ms_flushed": _stats(flushed1),
               "launch_ms_flushed_queued": _stats(queued1),
               "launch_ms_back_to_back": _stats(b2b1), "kernel": _lib.last_kernel()}
