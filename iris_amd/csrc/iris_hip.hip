@@ -443,8 +443,9 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     if (!strcmp(e, "skinny")) return (int)TILE_SKINNY;
     return -1;
   }();
-  if (forced_tile >= 0 && kind != TILE_DECODE && !(forced_tile == TILE_SKINNY && p.gather == GATHER_M && p.M_local % 64))
-    kind = forced_tile;
+  if (forced_tile >= 0 && kind != TILE_DECODE &&
+      !mfma_ineligible(p, in_dtype, out_dtype, tile_rows(forced_tile), tile_cols(forced_tile)))
+    kind = forced_tile;  // a tile the operands do not qualify for is not forced
   const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
   if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
