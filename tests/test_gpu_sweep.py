@@ -78,6 +78,33 @@ def test_every_build_bit_exact(dtype, tile, layout):
         assert_bits_equal(got, exp["C"][r], f"{kernel}: C in slot {r}")
 
 
+@pytest.mark.parametrize("tile,shape", [("256x256", (3000, 3088, 48)), ("128x128", (600, 400, 80)), ("128x128", (2300, 2064, 48)),
+                                        ("64x128", (48, 1168, 96))])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, FP8], ids=lambda d: NAMES[d])
+def test_atomic_variant_on_every_tile(dtype, tile, shape):
+    """The atomic epilogue deals the dwords of a tile out to the threads in its own order (one wave
+    instruction = 256 contiguous bytes); ragged edges in both directions, every tiled kernel."""
+    M, N, K = shape
+    W, rank = 3, 1
+    out_dtype = torch.bfloat16 if dtype == FP8 else dtype
+    ctx = iris.iris(1 << 27, num_ranks=W, rank=rank)
+    A, B = _operand((M, K), 17, dtype), _operand((K, N), 18, dtype)
+    before = [_operand((M, N), 60 + r, out_dtype, -40, 41) for r in range(W)]
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=out_dtype)
+    cfg = iris.FusedConfig(block_size_m=16, block_size_n=64, block_size_k=16, all_reduce_variant="atomic")
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    for r in range(W):
+        ctx.peer_view(dC, r).copy_(before[r])
+    ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, kernel_path="mfma", **_scales(dtype))
+    kernel = _lib.last_kernel()
+    assert kernel.startswith(f"mfma_{NAMES[dtype]}_{tile}"), kernel
+    scale = 0.5 if dtype == FP8 else 1.0
+    exp = oracle.matmul_all_reduce(A, B, before, rank, W, 16, 64, "atomic", out_dtype=out_dtype, scale=scale)
+    for r, got in enumerate(slot_copies(ctx, dC)):
+        assert_bits_equal(got, exp["C"][r], f"{kernel}: C in slot {r}")
+
+
 def _draw_shape(rng, dtype):
     ce = 16 if dtype == FP8 else 8  # elements per 16 bytes: K and N stay MFMA-eligible
     if rng.random() < 0.15:  # enough tiles for the 256x256 or the two-per-CU builds
