@@ -519,14 +519,17 @@ def test_c_abi_rejects_bad_arguments():
 # ------------------------------------------------------------------------------------------------
 # HIP graphs: a launch is one kernel node, so launch-bound loops can be captured and replayed
 # ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K,kernel", [(256, 384, 160, "128x128"), (32, 1168, 1360, "32x32"), (3072, 3072, 80, "256x256")])
 @pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
-def test_graph_replay_matches_eager(variant):
+def test_graph_replay_matches_eager(variant, M, N, K, kernel):
+    """Captured once, replayed four times with new operands: the tiled kernels and the decode kernel
+    (whose helper wave probes the peers' flags through heap bases that travel as kernel arguments)."""
     W, dtype = 4, torch.bfloat16
-    M, N, K = 256, 384, 160
     ctx = _ctx(W)
     B = randint_cpu((K, N), 21, dtype)
     peers = [randn_cpu((M, N), 200 + r, dtype) for r in range(W)]
-    cfg = iris.FusedConfig(block_size_m=64, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+    fbm = min(64, M)
+    cfg = iris.FusedConfig(block_size_m=fbm, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
     dA, dB = ctx.zeros((M, K), dtype=dtype), heap_tensor(ctx, B)
     dC = ctx.zeros((M, N), dtype=dtype)
     ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
@@ -557,7 +560,8 @@ def test_graph_replay_matches_eager(variant):
         graph.replay()
         torch.cuda.synchronize()
         ctx.check_status()
-        exp = oracle.matmul_all_reduce(A, B, peers, 0, W, 64, 64, variant, "fp32")
+        assert f"_{kernel}x" in _lib.last_kernel(), _lib.last_kernel()
+        exp = oracle.matmul_all_reduce(A, B, peers, 0, W, fbm, 64, variant, "fp32")
         assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"aux, replay {rep}")
         assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), f"flags, replay {rep}"
         got = slot_copies(ctx, dC)
