@@ -442,6 +442,44 @@ def test_unstaged_peer_flags_time_out():
 
 
 @pytest.mark.parametrize("M,N,K,variant", [(512, 384, 96, "one_shot"), (512, 384, 96, "two_shot"),
+                                           (32, 1168, 1360, "one_shot"), (3072, 3072, 80, "two_shot")])
+def test_peer_flags_raised_while_the_kernel_waits(M, N, K, variant):
+    """The normal case between real ranks: the peers' flags are not up yet when the kernel looks.  The
+    launch goes out with the peers' flags at zero; another stream raises them a little later.  The
+    kernel must have raised its own flags first, poll (bounded), and then sum what the peers
+    published - on the 128x128, the decode and the 256x256 kernel."""
+    W, rank, dtype = 4, 2, torch.bfloat16
+    ctx = _ctx(W, rank)
+    A, B = randint_cpu((M, K), 30, dtype), randint_cpu((K, N), 31, dtype)
+    peers = [randn_cpu((M, N), 400 + r, dtype) for r in range(W)]
+    fbm = 32 if M == 32 else 128
+    cfg = iris.FusedConfig(block_size_m=fbm, block_size_n=64, block_size_k=32, all_reduce_variant=variant)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    dC = ctx.zeros((M, N), dtype=dtype)
+    ws = ops.matmul_all_reduce_preamble(ctx, dC, dA, dB, config=cfg)
+    for r in range(W):
+        if r != rank:
+            ctx.peer_view(ws.aux_buffer, r).copy_(peers[r])
+            ctx.peer_view(ws.locks, r).zero_()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    ops.matmul_all_reduce(ctx, dC, dA, dB, async_op=True, config=cfg, workspace=ws)
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(2_000_000)  # the launch above is polling by now
+        for r in range(W):
+            if r != rank:
+                ctx.peer_view(ws.locks, r).fill_(1)
+    torch.cuda.synchronize()
+    ctx.check_status()  # no spin time-out
+    exp = oracle.matmul_all_reduce(A, B, peers, rank, W, fbm, 64, variant, "fp32")
+    assert torch.equal(ws.locks.cpu(), torch.from_numpy(exp["locks"])), "flags"
+    got = slot_copies(ctx, dC)
+    for r in range(W if variant == "two_shot" else 1):
+        slot = r if variant == "two_shot" else rank
+        assert_bits_equal(got[slot], exp["C"][slot], f"{_lib.last_kernel()} C in slot {slot}")
+
+
+@pytest.mark.parametrize("M,N,K,variant", [(512, 384, 96, "one_shot"), (512, 384, 96, "two_shot"),
                                            (32, 1168, 1360, "one_shot"), (3072, 3072, 80, "one_shot")])
 def test_unregistered_context_tensor_gives_the_same_bits(M, N, K, variant):
     """The kernels take the heap bases as kernel arguments when the host has registered the context
