@@ -1,4 +1,5 @@
-// Decode-sized problems (M <= 32 rows) of the flag-carrying operators: fused_decode_kernel.
+// Small outputs of the flag-carrying operators - decode-sized launches (M <= 32 rows) and, more
+// generally, outputs of at most two 32 x 32 tiles per CU: fused_decode_kernel.
 //
 // With so few rows the GEMM is a stream of B through the machine (config "fp8, M = 32, N = 8192,
 // K = 1024": 8 MB of B, 0.5 GFLOP) and the launch is a chain of memory round trips.  The tiled kernel
@@ -99,13 +100,16 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, 0, p.tiles_n, p.num_xcd);
+  // Tiles are numbered with the row tile running fastest, so that the workgroups that read the same
+  // columns of B (and those that share its 128-byte lines) are neighbours and land on one XCD.
+  const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, 0, p.tiles_m * p.tiles_n, p.num_xcd);
   if (tidx < 0) return;
 #ifdef IRIS_HIP_PHASE_STAMPS
   constexpr int it = 0;  // PHASE_STAMP records the first tile of a workgroup; there is only one here
 #endif
   PHASE_STAMP(0);
-  const int n0 = tidx * CFG::BN;
+  const int m0 = (tidx % p.tiles_m) * CFG::BM;
+  const int n0 = (tidx / p.tiles_m) * CFG::BN;
   const unsigned smem_base = __builtin_amdgcn_readfirstlane(lds_address(smem));
 
   // Heap bases: kernel arguments when the host knew them, else eight independent loads behind one
@@ -137,11 +141,11 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   const int npeers = solo ? 0 : p.world - 1;
   const int ftn = cdiv(p.N, p.flag_bn);
   const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
-  const int m1 = min(CFG::BM, p.M), n1 = min(n0 + CFG::BN, p.N);
-  const int fm_hi = (m1 - 1) / p.flag_bm;
+  const int m1 = min(m0 + CFG::BM, p.M), n1 = min(n0 + CFG::BN, p.N);
+  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
   const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
   const int nfn = fn_hi - fn_lo + 1;
-  const int nft = (fm_hi + 1) * nfn;  // flag tiles under this output tile
+  const int nft = (fm_hi - fm_lo + 1) * nfn;  // flag tiles under this output tile
 
   const bool helper = wave == CFG::NW;  // the wave that multiplies nothing
   const bool probing = helper && !solo && nft <= 64 && p.hb_in_args;
@@ -155,7 +159,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
     int t = 0;
     bool must_check = false;  // this lane's flag tile is one this rank reduces
     if (lane < nft) {
-      t = (lane / nfn) * ftn + fn_lo + lane % nfn;
+      t = (fm_lo + lane / nfn) * ftn + fn_lo + lane % nfn;
       must_check = p.all_owners || owner_of(p.epi, t, ftotal, p.world, p.rank) == p.rank;
     }
     const unsigned voff = must_check ? (unsigned)t * 4u : kInvalidOffset;
@@ -179,7 +183,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int q = lane + 64 * h, prow = q >> 2, pc = q & 3;
-        pv_off[h] = (prow < p.M && n0 + 8 * pc < p.N) ? (unsigned)(((long long)prow * p.s_cm + n0 + 8 * pc) * 2) : kInvalidOffset;
+        pv_off[h] = (m0 + prow < p.M && n0 + 8 * pc < p.N) ? (unsigned)(((long long)(m0 + prow) * p.s_cm + n0 + 8 * pc) * 2) : kInvalidOffset;
       }
       for (int i = 0; i < npeers; ++i) {
         const i32x4_t rs = make_rsrc_words(pbase[i] + aux_off);
@@ -204,7 +208,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
     int row, c;
     ATile::from_lds(i * kDmaBytes + lane * kChunkBytes, row, c);
     a_kb[i] = c * kChunkBytes;
-    a_voff[i] = row < p.M ? (unsigned)(row * p.s_am * ES + c * kChunkBytes) : kInvalidOffset;
+    a_voff[i] = m0 + row < p.M ? (unsigned)((m0 + row) * p.s_am * ES + c * kChunkBytes) : kInvalidOffset;
     if constexpr (BKC) {
       b_k[i] = c * kChunkBytes;
       b_voff[i] = n0 + row < p.N ? (unsigned)(row * p.s_bn * ES + c * kChunkBytes) : kInvalidOffset;
@@ -333,7 +337,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   // (this part of the launch is bound by instruction issue: twice the threads, half the time)
   const bool worker = tid < 256;
   const int row = (tid >> 3) & 31, c = tid & 7;
-  const int gm = row, gn = n0 + 4 * c;
+  const int gm = m0 + row, gn = n0 + 4 * c;
   const bool valid = worker && gm < p.M && gn < p.N;
   const long long eoff = valid ? ((long long)gm * p.s_cm + gn) * 2 : 0;
   u32x2_t own = {0, 0};
@@ -410,9 +414,9 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   wait_vmcnt<0>();
   __syncthreads();
   PHASE_STAMP(5);
-  raise_flags<CFG::BM, CFG::BN, CFG::NT, true>(p, 0, n0, tid);
+  raise_flags<CFG::BM, CFG::BN, CFG::NT, true>(p, m0, n0, tid);
   if (solo || have_peers) return;
-  wait_peer_flags<CFG::BM, CFG::BN, CFG::NT>(p, 0, n0, tid);
+  wait_peer_flags<CFG::BM, CFG::BN, CFG::NT>(p, m0, n0, tid);
   __syncthreads();
   PHASE_STAMP(6);
   if (reduces) reduce_and_store(false);
@@ -430,9 +434,9 @@ int launch_decode(FusedParams& p, int device, hipStream_t stream, const char* na
     if (e != hipSuccess) return (int)e;
     attr_set[device].store(true, std::memory_order_release);
   }
-  p.tiles_m = 1;
+  p.tiles_m = cdiv(p.M, CFG::BM);
   p.tiles_n = cdiv(p.N, CFG::BN);
-  int grid = p.tiles_n;
+  int grid = p.tiles_m * p.tiles_n;
   if (grid % p.num_xcd) grid += p.num_xcd - grid % p.num_xcd;  // the XCD mapping wants a multiple; surplus workgroups leave at once
   iris_host::set_last_kernel(name);
   hipLaunchKernelGGL((fused_decode_kernel<IN, BKC>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);

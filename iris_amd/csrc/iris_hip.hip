@@ -392,6 +392,16 @@ void heap_bases_from_registry(FusedParams& p, const int64_t* context_tensor) {
 unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
 #endif
 
+// Launches for the 32x32 kernel (decode_kernel.h): at most 32 rows, or any output small enough that
+// its 32x32 tiles make at most two rounds of one workgroup per CU.  Such outputs are a handful of
+// 128x128 tiles - 128 x 1024 is eight of them, on eight of 256 CUs - while the small tiles with K split
+// over the waves of a workgroup keep the whole chip busy (fp16, two-shot, eight ranks: 128x1024x4096 41 ->
+// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 14 us; from about 540 tiles on the tiled kernels win).
+bool decode_sized(const FusedParams& p, int cu_count) {
+  if (p.M <= 32) return true;
+  return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
+}
+
 int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
   g_last_error[0] = 0;
 #ifdef IRIS_HIP_PHASE_STAMPS
@@ -425,11 +435,11 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
   // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64-row tiles for decode-sized M, else
   // 128x128 - two workgroups per CU when there are more such tiles than CUs.  The flag-carrying operators
-  // with at most 32 rows take the latency-oriented 32x32 kernel (decode_kernel.h).
+  // take the latency-oriented 32x32 kernel (decode_kernel.h) for small outputs (decode_sized).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
-  else if (p.M <= 32 && epi_has_flags(p.epi) && p.gather == GATHER_NONE && p.world <= 8 && !p.bias) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count) && epi_has_flags(p.epi) && p.gather == GATHER_NONE && p.world <= 8 && !p.bias) kind = TILE_DECODE;
   else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
   // IRIS_HIP_TILE = big | small | small2 | skinny overrides the choice among the tiled kernels (a tuning
