@@ -137,13 +137,15 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   // Slots of the peers in ascending rank order, own rank skipped.
   auto peer_slot = [&](int i) { return i < p.rank ? i : i + 1; };
 
-  const bool solo = !p.sum_peers || p.world == 1;
+  const bool flagged = epi_has_flags(p.epi);  // else: plain store, all-gather or atomic epilogue - no aux, no flags
+  const bool solo = !flagged || !p.sum_peers || p.world == 1;
   const int npeers = solo ? 0 : p.world - 1;
-  const int ftn = cdiv(p.N, p.flag_bn);
-  const int ftotal = cdiv(p.M, p.flag_bm) * ftn;
+  const int fbm = flagged ? p.flag_bm : CFG::BM, fbn = flagged ? p.flag_bn : CFG::BN;  // no flag tiles without flags
+  const int ftn = cdiv(p.N, fbn);
+  const int ftotal = cdiv(p.M, fbm) * ftn;
   const int m1 = min(m0 + CFG::BM, p.M), n1 = min(n0 + CFG::BN, p.N);
-  const int fm_lo = m0 / p.flag_bm, fm_hi = (m1 - 1) / p.flag_bm;
-  const int fn_lo = n0 / p.flag_bn, fn_hi = (n1 - 1) / p.flag_bn;
+  const int fm_lo = m0 / fbm, fm_hi = (m1 - 1) / fbm;
+  const int fn_lo = n0 / fbn, fn_hi = (n1 - 1) / fbn;
   const int nfn = fn_hi - fn_lo + 1;
   const int nft = (fm_hi - fm_lo + 1) * nfn;  // flag tiles under this output tile
 
@@ -348,10 +350,33 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
       const float* part = (const float*)(smem + CFG::OPERANDS + w * CFG::WAVE_BYTES) + row * CFG::RED_STRIDE + 4 * c;
       s4 += *(const LDS_AS f32x4_t*)(LDS_AS const char*)((const char*)part);
     }
-    own.x = Out::pack(s4.x * p.scale, s4.y * p.scale);
-    own.y = Out::pack(s4.z * p.scale, s4.w * p.scale);
+    // per-row bias of the operators that have one (added in fp32, before the cast)
+    const float badd = (p.bias && gm < p.M) ? load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype) : 0.f;
+    own.x = Out::pack(s4.x * p.scale + badd, s4.y * p.scale + badd);
+    own.y = Out::pack(s4.z * p.scale + badd, s4.w * p.scale + badd);
   }
   const unsigned long long c_own = (unsigned long long)p.C;
+  if (!flagged) {
+    // The operators without flags: the tile goes to C (plain GEMM), to every rank's gathered output at
+    // this rank's row block (iris/mem/triton/context.py:841-864), or is added into every rank's C
+    // (iris/mem/triton/context.py:689-702; two packed dwords per piece).
+    if (valid) {
+      const long long goff = ((long long)(gm + p.row_offset) * p.s_cm + gn) * 2;
+      if (p.epi == EPI_ATOMIC) {
+        for (int pr = 0; pr < p.world; ++pr) {
+          char* dst = (char*)(in_slot(c_own, pr) + goff);
+          atomic_add_packed<Out>(dst, own.x);
+          atomic_add_packed<Out>(dst + 4, own.y);
+        }
+      } else if (p.epi == EPI_ALL_GATHER) {
+        for (int pr = 0; pr < p.world; ++pr) __builtin_nontemporal_store(own, (u32x2_t*)(in_slot(c_own, pr) + goff));
+      } else {
+        __builtin_nontemporal_store(own, (u32x2_t*)(c_own + goff));
+      }
+    }
+    PHASE_STAMP(4);
+    return;
+  }
   int owner = p.rank;
   if (p.epi != EPI_ONE_SHOT) owner = owner_of(p.epi, (gm / p.flag_bm) * ftn + gn / p.flag_bn, ftotal, p.world, p.rank);
   const bool reduces = valid && (p.all_owners || owner == p.rank);

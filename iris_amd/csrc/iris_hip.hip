@@ -439,7 +439,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
-  else if (decode_sized(p, facts->cu_count) && epi_has_flags(p.epi) && p.gather == GATHER_NONE && p.world <= 8 && !p.bias) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count) && p.gather == GATHER_NONE && p.world <= 8) kind = TILE_DECODE;
   else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
   // IRIS_HIP_TILE = big | small | small2 | skinny overrides the choice among the tiled kernels (a tuning

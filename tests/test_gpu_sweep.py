@@ -80,12 +80,13 @@ def test_every_build_bit_exact(dtype, tile, layout):
         assert_bits_equal(got, exp["C"][r], f"{kernel}: C in slot {r}")
 
 
-@pytest.mark.parametrize("tile,shape", [("256x256", (3000, 3088, 48)), ("128x128", (600, 400, 80)), ("128x128", (2300, 2064, 48)),
-                                        ("64x128", (48, 1168, 96))])
+@pytest.mark.parametrize("tile,shape", [("256x256", (3000, 3088, 48)), ("128x128", (1300, 1040, 80)), ("128x128", (2300, 2064, 48)),
+                                        ("64x128", (48, 8336, 96)), ("32x32", (600, 400, 80)), ("32x32", (48, 1168, 96))])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, FP8], ids=lambda d: NAMES[d])
 def test_atomic_variant_on_every_tile(dtype, tile, shape):
     """The atomic epilogue deals the dwords of a tile out to the threads in its own order (one wave
-    instruction = 256 contiguous bytes); ragged edges in both directions, every tiled kernel."""
+    instruction = 256 contiguous bytes); ragged edges in both directions, every tiled kernel and the
+    small-output kernel."""
     M, N, K = shape
     W, rank = 3, 1
     out_dtype = torch.bfloat16 if dtype == FP8 else dtype
