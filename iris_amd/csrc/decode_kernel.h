@@ -1,5 +1,6 @@
-// Small outputs of the flag-carrying operators - decode-sized launches (M <= 32 rows) and, more
-// generally, outputs of at most two 32 x 32 tiles per CU: fused_decode_kernel.
+// Small outputs - decode-sized launches (M <= 32 rows) and, more generally, outputs of at most two
+// 32 x 32 tiles per CU - of every operator that does not gather A: fused_decode_kernel.  The description
+// follows the flag-carrying operators; the others leave after the partial tiles have met.
 //
 // With so few rows the GEMM is a stream of B through the machine (config "fp8, M = 32, N = 8192,
 // K = 1024": 8 MB of B, 0.5 GFLOP) and the launch is a chain of memory round trips.  The tiled kernel

@@ -434,8 +434,8 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
 
   // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
   // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64-row tiles for decode-sized M, else
-  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  The flag-carrying operators
-  // take the latency-oriented 32x32 kernel (decode_kernel.h) for small outputs (decode_sized).
+  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Small outputs (decode_sized)
+  // whose A is not gathered take the latency-oriented 32x32 kernel (decode_kernel.h).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
