@@ -433,14 +433,18 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   hipStream_t s = (hipStream_t)stream;
 
   // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
-  // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64-row tiles for decode-sized M, else
+  // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64x128 tiles for M <= 64 and for outputs
+  // that are at most one such tile per CU (128x128 tiles would leave half the chip idle: fp16, two-shot,
+  // eight ranks, 512x4096x512 21.3 -> 15.7 us, 256x8192x4096 48.5 -> 42.3 us, 1024x2048x512 21.0 -> 15.9 us), else
   // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Small outputs (decode_sized)
   // whose A is not gathered take the latency-oriented 32x32 kernel (decode_kernel.h).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
   else if (decode_sized(p, facts->cu_count) && p.gather == GATHER_NONE && p.world <= 8) kind = TILE_DECODE;
-  else if (p.M <= 64 && !(p.gather == GATHER_M && p.M_local % 64)) kind = TILE_SKINNY;
+  else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
+           !(p.gather == GATHER_M && p.M_local % 64))
+    kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
   // IRIS_HIP_TILE = big | small | small2 | skinny overrides the choice among the tiled kernels (a tuning
   // aid; results do not depend on the tile shape beyond the order of the fp32 sums over K).

@@ -21,11 +21,12 @@ FP8 = torch.float8_e4m3fn
 NAMES = {torch.bfloat16: "bf16", torch.float16: "f16", FP8: "fp8"}
 
 # Shapes that make the host pick each tile shape on a 256-CU part: >= 136 tiles of 256x256 (big), at
-# most 256 tiles of 128x128 (small), more than that (small2, two workgroups per CU), M <= 64 (skinny);
+# most 256 tiles of 128x128 but more than 256 of 64x128 (small), more than 256 of 128x128 (small2, two
+# workgroups per CU), M <= 64 or at most 256 tiles of 64x128 (skinny);
 # outputs of at most 512 tiles of 32x32 take the small-output kernel (one row tile, and six of them).
 TILE_SHAPES = {
     "256x256": (3072, 3072, 80),
-    "128x128s": (1280, 1024, 208),   # 128-byte K steps
+    "128x128s": (1280, 3072, 208),   # 128-byte K steps
     "128x128d": (2304, 2048, 80),    # 64-byte K steps, two workgroups per CU
     "64x128": (48, 8320, 336),
     "32x32": (32, 1168, 1360),       # at most 32 rows: K in 1024-byte chunks (2 or 3 here)
@@ -80,7 +81,7 @@ def test_every_build_bit_exact(dtype, tile, layout):
         assert_bits_equal(got, exp["C"][r], f"{kernel}: C in slot {r}")
 
 
-@pytest.mark.parametrize("tile,shape", [("256x256", (3000, 3088, 48)), ("128x128", (1300, 1040, 80)), ("128x128", (2300, 2064, 48)),
+@pytest.mark.parametrize("tile,shape", [("256x256", (3000, 3088, 48)), ("128x128", (1300, 3088, 80)), ("128x128", (2300, 2064, 48)),
                                         ("64x128", (48, 8336, 96)), ("32x32", (600, 400, 80)), ("32x32", (48, 1168, 96))])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, FP8], ids=lambda d: NAMES[d])
 def test_atomic_variant_on_every_tile(dtype, tile, shape):
