@@ -1,5 +1,5 @@
 // Small outputs - decode-sized launches (M <= 32 rows) and, more generally, outputs of at most two
-// 32 x 32 tiles per CU - of every operator that does not gather A: fused_decode_kernel.  The description
+// 32 x 32 tiles per CU - of every operator: fused_decode_kernel.  The description
 // follows the flag-carrying operators; the others leave after the partial tiles have met.
 //
 // With so few rows the GEMM is a stream of B through the machine (config "fp8, M = 32, N = 8192,
@@ -204,6 +204,17 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   // ---- operand loaders ---------------------------------------------------------------------------
   // Per lane and load: byte offset inside the operand and the k byte (A, K-contiguous B) or k row
   // (row-major B) it covers relative to the wave's first k of a chunk.
+  // A gathered from the ranks' slots (iris/mem/triton/context.py:866-888): by rows, the tile's 32 rows
+  // come from one slot (the host admits row gathering only for whole tiles per slot); by columns, the
+  // slot changes along K and is looked up per chunk below.
+  const unsigned long long a_own = (unsigned long long)p.A;
+  unsigned long long a_base = a_own;
+  int a_row0 = m0;
+  if (p.gather == GATHER_M) {
+    const int src = m0 / p.M_local;
+    a_base = in_slot(a_own, src);
+    a_row0 = m0 - src * p.M_local;
+  }
   unsigned a_voff[LOADS / 2], b_voff[LOADS / 2];
   int a_kb[LOADS / 2], b_k[LOADS / 2];
 #pragma unroll
@@ -211,7 +222,7 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
     int row, c;
     ATile::from_lds(i * kDmaBytes + lane * kChunkBytes, row, c);
     a_kb[i] = c * kChunkBytes;
-    a_voff[i] = m0 + row < p.M ? (unsigned)((m0 + row) * p.s_am * ES + c * kChunkBytes) : kInvalidOffset;
+    a_voff[i] = m0 + row < p.M ? (unsigned)((a_row0 + row) * p.s_am * ES + c * kChunkBytes) : kInvalidOffset;
     if constexpr (BKC) {
       b_k[i] = c * kChunkBytes;
       b_voff[i] = n0 + row < p.N ? (unsigned)(row * p.s_bn * ES + c * kChunkBytes) : kInvalidOffset;
@@ -222,7 +233,8 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
       b_voff[i] = n0 + cc * CE < p.N ? (unsigned)(krow * p.s_bk * ES + cc * kChunkBytes) : kInvalidOffset;
     }
   }
-  const i32x4_t ra = make_rsrc_words((unsigned long long)p.A);
+  i32x4_t ra = make_rsrc_words(a_base);
+  const int klb = p.K_local * ES;  // bytes of K one slot holds when A is gathered along K (a multiple of QB)
   const i32x4_t rb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)n0 * (BKC ? p.s_bn : 1) * ES);
   const int kbytes = p.K * ES;
   const int nchunks = cdiv(kbytes, CFG::NW * CFG::QB);
@@ -230,9 +242,15 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
     const unsigned region = smem_base + CFG::OPERANDS + (ch & 1) * CFG::BUF_BYTES + wave * CFG::WAVE_BYTES;
     const int kb0 = (ch * CFG::NW + wave) * CFG::QB;  // first k byte of the wave in this chunk
     const int left = kbytes - kb0;                      // k bytes of this wave's share that exist
+    unsigned a_soff = (unsigned)kb0;
+    if (p.gather == GATHER_K) {  // the wave's 256 bytes of K lie in one slot
+      const int src = min(kb0 / klb, p.world - 1);
+      ra = make_rsrc_words(in_slot(a_own, src));
+      a_soff = (unsigned)(kb0 - src * klb);
+    }
 #pragma unroll
     for (int i = 0; i < LOADS / 2; ++i)
-      dma16(ra, region + i * kDmaBytes, a_kb[i] < left ? a_voff[i] : kInvalidOffset, (unsigned)kb0);
+      dma16(ra, region + i * kDmaBytes, a_kb[i] < left ? a_voff[i] : kInvalidOffset, a_soff);
     const unsigned b_soff = __builtin_amdgcn_readfirstlane(BKC ? (unsigned)kb0 : (unsigned)((long long)(kb0 / ES) * p.s_bk * ES));
 #pragma unroll
     for (int i = 0; i < LOADS / 2; ++i) {

@@ -401,6 +401,14 @@ bool decode_sized(const FusedParams& p, int cu_count) {
   if (p.M <= 32) return true;
   return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
 }
+// ... and whose A that kernel can fetch: not gathered, gathered by rows in whole 32-row tiles per slot, or
+// gathered along K with every wave's 256 bytes of K inside one slot.
+bool decode_gather_ok(const FusedParams& p, int in_dtype) {
+  const int es = in_dtype == IRIS_HIP_FP8_E4M3 ? 1 : 2;
+  if (p.gather == GATHER_M) return p.M_local % 32 == 0;
+  if (p.gather == GATHER_K) return ((long long)p.K_local * es) % 256 == 0;
+  return true;
+}
 
 int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
   g_last_error[0] = 0;
@@ -437,11 +445,11 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   // that are at most one such tile per CU (128x128 tiles would leave half the chip idle: fp16, two-shot,
   // eight ranks, 512x4096x512 21.3 -> 15.7 us, 256x8192x4096 48.5 -> 42.3 us, 1024x2048x512 21.0 -> 15.9 us), else
   // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Small outputs (decode_sized)
-  // whose A is not gathered take the latency-oriented 32x32 kernel (decode_kernel.h).
+  // take the latency-oriented 32x32 kernel (decode_kernel.h).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
-  else if (decode_sized(p, facts->cu_count) && p.gather == GATHER_NONE && p.world <= 8) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
   else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
            !(p.gather == GATHER_M && p.M_local % 64))
     kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own

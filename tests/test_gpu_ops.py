@@ -309,6 +309,38 @@ def test_all_gather_matmul_rows_and_bias():
         assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B, bias=bias, gather_dim=0), path)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn], ids=["bf16", "fp8"])
+@pytest.mark.parametrize("gather_dim,W,rank,M,Kl,N", [(1, 8, 5, 80, 128, 272), (1, 2, 0, 200, 384, 144), (1, 3, 2, 32, 512, 1168),
+                                                        (0, 4, 1, 32, 144, 528), (0, 8, 7, 64, 1360, 80)])
+def test_all_gather_matmul_small_outputs(dtype, gather_dim, W, rank, M, Kl, N):
+    """Small outputs take the 32x32 kernel also when A is gathered: along K the slot changes between the
+    256-byte pieces of K that the waves own (K_local a multiple of 256 bytes), along M between row
+    tiles (M here is the rows per slot); with and without the row bias, integer data, every bit."""
+    fp8 = dtype == torch.float8_e4m3fn
+    if fp8 and gather_dim == 1:
+        Kl *= 2  # 256 bytes are 256 e4m3 values
+    out_dtype = torch.bfloat16 if fp8 else dtype
+    ctx = _ctx(W, rank)
+    shards = [randint_cpu((M, Kl), 500 + r, torch.float32, -3, 4).to(dtype) for r in range(W)]
+    Kt = Kl * W if gather_dim == 1 else Kl
+    rows = M if gather_dim == 1 else M * W
+    B = randint_cpu((Kt, N), 520, torch.float32, -3, 4).to(dtype)
+    bias = randint_cpu((rows,), 521, out_dtype, -8, 9) if (rank % 2) else None
+    dA = ctx.zeros((M, Kl), dtype=dtype)
+    for r in range(W):
+        ctx.peer_view(dA, r).copy_(shards[r])
+    dB = heap_tensor(ctx, B)
+    dbias = heap_tensor(ctx, bias) if bias is not None else None
+    out = ctx.zeros((rows, N), dtype=out_dtype)
+    cfg = iris.FusedConfig(block_size_m=16, block_size_n=16, block_size_k=16)
+    kw = dict(scale_a=0.5, scale_b=2.0) if fp8 else {}
+    ops.all_gather_matmul(ctx, out, dA, dB, bias=dbias, config=cfg, gather_dim=gather_dim, **kw)
+    kernel = _lib.last_kernel()
+    assert "_32x32x" in kernel, kernel
+    exp = oracle.all_gather_matmul(shards, B, bias=bias, gather_dim=gather_dim, out_dtype=out_dtype, scale=1.0)
+    assert_bits_equal(out.cpu(), exp, f"{kernel} gather_dim={gather_dim} bias={bias is not None}")
+
+
 def test_all_gather_matmul_random_via_namespace():
     W, rank, dtype = 4, 0, torch.float16
     M, K_local, N = 256, 64, 128
