@@ -30,8 +30,9 @@
 
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-template <int IN_, bool B_KCONTIG_>
+template <int IN_, bool B_KCONTIG_, int QB_ = 256>
 struct DecodeCfg {
+  static_assert(QB_ == 128 || QB_ == 256, "a wave owns 128 or 256 bytes of K per chunk");
   static constexpr int IN = IN_;
   static constexpr bool B_KCONTIG = B_KCONTIG_;
   static constexpr int ES = (IN_ == IN_FP8) ? 1 : 2;
@@ -40,16 +41,16 @@ struct DecodeCfg {
   static constexpr int NFRAG = (IN_ == IN_FP8) ? 2 : 1;
   static constexpr int BM = 32, BN = 32, NW = 4;  // NW waves multiply
   static constexpr int NT = 64 * (NW + 1);         // ... and one more probes flags and fetches the peers' tiles
-  static constexpr int QB = 256;                  // bytes of K one wave owns per chunk
+  static constexpr int QB = QB_;                  // bytes of K one wave owns per chunk
   static constexpr int KQ = QB / ES;              // ... in elements
   static constexpr int CHUNK = NW * KQ;           // k elements per chunk of the workgroup
   static constexpr int NSL = KQ / KM;             // MFMAs per wave and chunk
   static constexpr int RBB = B_KCONTIG ? QB : BN * ES;  // bytes per row of a wave's B region
-  static constexpr int A_BYTES = BM * QB;         // 8 KiB
-  static constexpr int B_BYTES = 8192;            // [32 n][256 B] or [KQ k][32 * ES B]
+  static constexpr int A_BYTES = BM * QB;         // 8 KiB (4 KiB with 128-byte shares)
+  static constexpr int B_BYTES = BN * QB;         // [32 n][QB B] or [KQ k][32 * ES B]
   static constexpr int WAVE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int BUF_BYTES = NW * WAVE_BYTES;       // one chunk of the workgroup: 64 KiB
-  static constexpr int LOADS = WAVE_BYTES / kDmaBytes;    // direct-to-LDS loads per wave and chunk: 16
+  static constexpr int BUF_BYTES = NW * WAVE_BYTES;       // one chunk of the workgroup: 64 KiB (32 KiB)
+  static constexpr int LOADS = WAVE_BYTES / kDmaBytes;    // direct-to-LDS loads per wave and chunk: 16 (8)
   static constexpr int RED_STRIDE = 36;                   // floats per row of a partial accumulator
   static constexpr int MAX_PEERS = 7;
   static constexpr int PEER_BYTES = BM * BN * 2;          // one peer's 32 x 32 tile of 16-bit values
@@ -58,8 +59,8 @@ struct DecodeCfg {
   static constexpr int PROBE_AREA = PEER_AREA + MAX_PEERS * PEER_BYTES;
   static constexpr int WORD_AREA = PROBE_AREA + MAX_PEERS * 256;
   static constexpr int OPERANDS = WORD_AREA + 256;  // 16 KiB
-  static constexpr int SMEM_BYTES = OPERANDS + 2 * BUF_BYTES;
-  static_assert(NW * BM * RED_STRIDE * 4 <= BUF_BYTES && BM * RED_STRIDE * 4 <= A_BYTES, "partials reuse operand space");
+  static constexpr int SMEM_BYTES = OPERANDS + 2 * BUF_BYTES;  // 144 KiB: one workgroup per CU; 80 KiB: two
+  static_assert(BM * RED_STRIDE * 4 <= WAVE_BYTES, "a wave's partial tile reuses its own operand region");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
 };
 
@@ -85,9 +86,9 @@ __device__ __forceinline__ void dma16_system(i32x4_t rsrc, unsigned lds_base, un
                : "memory");
 }
 
-template <int IN, bool BKC>
+template <int IN, bool BKC, int QB>
 __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_in) {
-  using CFG = DecodeCfg<IN, BKC>;
+  using CFG = DecodeCfg<IN, BKC, QB>;
   using Out = typename OutOf<IN>::type;
   using ATile = RowTile<CFG::QB>;
   constexpr int ES = CFG::ES, CE = CFG::CE, NFRAG = CFG::NFRAG, LOADS = CFG::LOADS, MAXP = CFG::MAX_PEERS;
@@ -238,12 +239,12 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   const i32x4_t rb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)n0 * (BKC ? p.s_bn : 1) * ES);
   const int kbytes = p.K * ES;
   const int nchunks = cdiv(kbytes, CFG::NW * CFG::QB);
-  auto issue_chunk = [&](int ch) {  // this wave's 16 loads of chunk ch
+  auto issue_chunk = [&](int ch) {  // this wave's loads of chunk ch
     const unsigned region = smem_base + CFG::OPERANDS + (ch & 1) * CFG::BUF_BYTES + wave * CFG::WAVE_BYTES;
     const int kb0 = (ch * CFG::NW + wave) * CFG::QB;  // first k byte of the wave in this chunk
     const int left = kbytes - kb0;                      // k bytes of this wave's share that exist
     unsigned a_soff = (unsigned)kb0;
-    if (p.gather == GATHER_K) {  // the wave's 256 bytes of K lie in one slot
+    if (p.gather == GATHER_K) {  // the wave's bytes of K lie in one slot
       const int src = min(kb0 / klb, p.world - 1);
       ra = make_rsrc_words(in_slot(a_own, src));
       a_soff = (unsigned)(kb0 - src * klb);
@@ -467,13 +468,13 @@ __global__ void __launch_bounds__(320) fused_decode_kernel(const FusedParams p_i
   PHASE_STAMP(7);
 }
 
-template <int IN, bool BKC>
+template <int IN, bool BKC, int QB>
 int launch_decode(FusedParams& p, int device, hipStream_t stream, const char* name) {
-  using CFG = DecodeCfg<IN, BKC>;
+  using CFG = DecodeCfg<IN, BKC, QB>;
   static std::atomic<bool> attr_set[64];
   if (device < 0 || device >= 64) return iris_host::fail("device index %d out of range", device);
   if (!attr_set[device].load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_decode_kernel<IN, BKC>,
+    hipError_t e = hipFuncSetAttribute((const void*)fused_decode_kernel<IN, BKC, QB>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
     if (e != hipSuccess) return (int)e;
     attr_set[device].store(true, std::memory_order_release);
@@ -483,6 +484,6 @@ int launch_decode(FusedParams& p, int device, hipStream_t stream, const char* na
   int grid = p.tiles_m * p.tiles_n;
   if (grid % p.num_xcd) grid += p.num_xcd - grid % p.num_xcd;  // the XCD mapping wants a multiple; surplus workgroups leave at once
   iris_host::set_last_kernel(name);
-  hipLaunchKernelGGL((fused_decode_kernel<IN, BKC>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
+  hipLaunchKernelGGL((fused_decode_kernel<IN, BKC, QB>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
   return (int)hipGetLastError();
 }
