@@ -8,7 +8,9 @@
 // one is built for latency instead:
 //   * 32 x 32 output tiles, so N / 32 workgroups (256 for N = 8192) pull B at the same time; the
 //     workgroups that share a 128-byte line of B sit on the same XCD;
-//   * the four waves split K: in every chunk of 1024 bytes of K each wave owns 256 bytes, loads exactly
+//   * the four waves split K: in every chunk of 1024 bytes of K each wave owns 256 bytes (512 and 128 in the
+//     build the host takes when there are more tiles than CUs - two workgroups then share a CU - or when K
+//     is short), loads exactly
 //     the operand bytes it multiplies (direct-to-LDS, into a region no other wave touches) and waits for
 //     nothing but its own loads - the K phase has no workgroup barrier; problems whose K fits one or two
 //     chunks (K <= 2048 bytes) have every operand load in flight from the first instruction on;
