@@ -13,7 +13,7 @@ from typing import Optional, Tuple
 import torch
 
 from .. import _lib
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ..ops._common import current_stream, dtype_code, iris_launch, ptr, require_gpu_tensors
 from .config import Config
 from .utils import ReduceOp, extract_group_info
@@ -136,8 +136,9 @@ def all_reduce(output_tensor, input_tensor, ctx, op=None, group=None, async_op=F
         workspace = all_reduce_preamble(output_tensor, input_tensor, ctx, config=config, workspace=workspace)
 
     head, rank_global = _launch_head(ctx, output_tensor, input_tensor, config, group)
-    log_rank(logging.DEBUG, "ccl.all_reduce: shape=(%d,%d) dtype=%s variant=%s", M, N, input_tensor.dtype, variant,
-             rank=rank_global, num_ranks=ctx.get_num_ranks())
+    if debug_on():
+        log_rank(logging.DEBUG, "ccl.all_reduce: shape=(%d,%d) dtype=%s variant=%s", M, N, input_tensor.dtype, variant,
+                 rank=rank_global, num_ranks=ctx.get_num_ranks())
     require_gpu_tensors(ctx, input_tensor=input_tensor, output_tensor=output_tensor)
     iris_launch(
         "iris_hip_all_reduce", (config.comm_sms,), *head,

@@ -6,7 +6,7 @@ iris/ccl/triton/reduce_scatter.py:143-192.
 
 import logging
 
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ..ops._common import current_stream, dtype_code, iris_launch, require_gpu_tensors
 from .all_reduce import _check_tensors, _launch_head
 from .config import Config
@@ -43,8 +43,9 @@ def reduce_scatter(output_tensor, input_tensor, ctx, op=None, group=None, async_
         )
     code = dtype_code(input_tensor.dtype)
     head, rank_global = _launch_head(ctx, output_tensor, input_tensor, config, group)
-    log_rank(logging.DEBUG, "ccl.reduce_scatter: shape=(%d,%d) dtype=%s", M, N, input_tensor.dtype,
-             rank=rank_global, num_ranks=ctx.get_num_ranks())
+    if debug_on():
+        log_rank(logging.DEBUG, "ccl.reduce_scatter: shape=(%d,%d) dtype=%s", M, N, input_tensor.dtype,
+                 rank=rank_global, num_ranks=ctx.get_num_ranks())
     require_gpu_tensors(ctx, input_tensor=input_tensor, output_tensor=output_tensor)
     iris_launch(
         "iris_hip_reduce_scatter", (config.comm_sms,), *head,

@@ -46,6 +46,11 @@ def log_rank(level, msg, *args, rank=None, num_ranks=None):
         logger.log(level, msg, *args, extra=extra, stacklevel=2)
 
 
+def debug_on():
+    """Whether DEBUG records are emitted: lets a hot path skip building a record's arguments."""
+    return logger.isEnabledFor(logging.DEBUG)
+
+
 def set_logger_level(level):
     """Set the level of the "iris" logger (iris.DEBUG, iris.INFO, iris.WARNING, iris.ERROR)."""
     logger.setLevel(level)

@@ -1,21 +1,23 @@
 """Plumbing shared by the operator wrappers: element-type codes, the launch seam, argument checks."""
 
-import ctypes
 import logging
 
 import torch
 
 from .. import _lib
 from ..host.hip import error_string
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 
 _DTYPE_CODES = {
     torch.bfloat16: _lib.BF16,
     torch.float16: _lib.FP16,
     torch.float32: _lib.FP32,
 }
-if hasattr(torch, "float8_e4m3fn"):
-    _DTYPE_CODES[torch.float8_e4m3fn] = _lib.FP8_E4M3
+_FP8 = getattr(torch, "float8_e4m3fn", None)
+if _FP8 is not None:
+    _DTYPE_CODES[_FP8] = _lib.FP8_E4M3
+
+_ENTRY_POINTS = {}  # name -> bound foreign function (prototypes applied by _lib.library())
 
 _PATHS = {"auto": _lib.PATH_AUTO, "mfma": _lib.PATH_MFMA, "generic": _lib.PATH_GENERIC}
 _ACC = {"fp32": _lib.ACC_FP32, "reference": _lib.ACC_REFERENCE}
@@ -29,7 +31,7 @@ def dtype_code(dtype):
 
 
 def is_fp8(dtype):
-    return hasattr(torch, "float8_e4m3fn") and dtype == torch.float8_e4m3fn
+    return _FP8 is not None and dtype == _FP8
 
 
 def path_code(path):
@@ -57,23 +59,29 @@ def require_gpu_tensors(shmem, **tensors):
 
 
 def ptr(t):
-    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+    """Device address of a tensor as the prototypes' void* takes it: a plain integer, None for no tensor
+    (the operators are called once per few microseconds for small shapes; a ctypes object per argument
+    was a tenth of the call)."""
+    return t.data_ptr() if t is not None else None
 
 
 def current_stream(shmem):
     """The raw HIP stream torch would launch on for the context's device right now (honours
     `with torch.cuda.stream(...)` and graph capture)."""
-    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(shmem.get_device_id()))
+    return torch._C._cuda_getCurrentRawStream(shmem.get_device_id())
 
 
 def iris_launch(entry_name, grid, *args, algorithm, rank, dtype=None):
     """Launch seam: the reference launches `kernel_fn[grid](*args)` here
     (iris/host/tracing/kernel_artifacts.py:54-83); this calls the C entry point of the same operator
     and turns a non-zero hipError_t into RuntimeError the way gpu_try does."""
-    log_rank(logging.DEBUG, "iris_launch: algorithm=%s kernel=%s grid=%s rank=%d", algorithm, entry_name, grid,
-             rank, rank=rank)
-    lib = _lib.library()
-    err = getattr(lib, entry_name)(*args)
+    if debug_on():
+        log_rank(logging.DEBUG, "iris_launch: algorithm=%s kernel=%s grid=%s rank=%d", algorithm, entry_name, grid,
+                 rank, rank=rank)
+    entry = _ENTRY_POINTS.get(entry_name)
+    if entry is None:
+        entry = _ENTRY_POINTS[entry_name] = getattr(_lib.library(), entry_name)
+    err = entry(*args)
     if err != 0:
         detail = _lib.last_error()
         text = detail if detail else error_string(err)

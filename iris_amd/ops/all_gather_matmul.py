@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ._common import current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr, require_gpu_tensors
 from .config import FusedConfig
 from .workspace import FusedWorkspace
@@ -82,8 +82,9 @@ def all_gather_matmul(
     else:
         M_local, K_local = A_sharded.shape
         M = M_local * world_size
-    log_rank(logging.DEBUG, "all_gather_matmul: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M, N, K, A_sharded.dtype, rank,
-             world_size, rank=rank, num_ranks=world_size)
+    if debug_on():
+        log_rank(logging.DEBUG, "all_gather_matmul: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M, N, K, A_sharded.dtype, rank,
+                 world_size, rank=rank, num_ranks=world_size)
 
     if gather_dim == 1:
         expected_K = world_size * K_local

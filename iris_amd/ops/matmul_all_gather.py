@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ._common import current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr, require_gpu_tensors
 from .config import FusedConfig
 from .workspace import FusedWorkspace
@@ -64,8 +64,9 @@ def matmul_all_gather(
     K2, N = B.shape
     world_size = shmem.get_num_ranks()
     rank = shmem.get_rank()
-    log_rank(logging.DEBUG, "matmul_all_gather: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M_local * world_size, N, K,
-             A.dtype, rank, world_size, rank=rank, num_ranks=world_size)
+    if debug_on():
+        log_rank(logging.DEBUG, "matmul_all_gather: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M_local * world_size, N, K,
+                 A.dtype, rank, world_size, rank=rank, num_ranks=world_size)
     assert K == K2, f"Inner dimensions must match: A has K={K}, B has K={K2}"
     M = M_local * world_size
     assert output_tensor.shape == (M, N), f"Output must be ({M}, {N}), got {output_tensor.shape}"

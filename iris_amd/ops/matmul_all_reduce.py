@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ._common import (acc_code, current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr,
                       require_gpu_tensors, stage_idle_peers)
 from .config import FusedConfig
@@ -132,8 +132,9 @@ def matmul_all_reduce(
     stride_cm, stride_cn = C.stride()
     rank = shmem.get_rank()
     world_size = shmem.get_num_ranks()
-    log_rank(logging.DEBUG, "matmul_all_reduce: shape=(%d,%d,%d) dtype=%s variant=%s rank=%d/%d", M, N, K, A.dtype,
-             config.all_reduce_variant, rank, world_size, rank=rank, num_ranks=world_size)
+    if debug_on():
+        log_rank(logging.DEBUG, "matmul_all_reduce: shape=(%d,%d,%d) dtype=%s variant=%s rank=%d/%d", M, N, K, A.dtype,
+                 config.all_reduce_variant, rank, world_size, rank=rank, num_ranks=world_size)
     if config.all_reduce_variant not in _VARIANT_CODES:
         config.validate(world_size=world_size)
         raise NotImplementedError(

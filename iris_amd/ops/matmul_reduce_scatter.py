@@ -10,7 +10,7 @@ from typing import Optional
 
 import torch
 
-from ..host.logging import log_rank
+from ..host.logging import debug_on, log_rank
 from ._common import (acc_code, current_stream, dtype_code, iris_launch, is_fp8, path_code, ptr,
                       require_gpu_tensors, stage_idle_peers)
 from .config import FusedConfig
@@ -122,8 +122,9 @@ def matmul_reduce_scatter(
     N = B.shape[1]
     rank = shmem.get_rank()
     world_size = shmem.get_num_ranks()
-    log_rank(logging.DEBUG, "matmul_reduce_scatter: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M, N, K, A.dtype, rank,
-             world_size, rank=rank, num_ranks=world_size)
+    if debug_on():
+        log_rank(logging.DEBUG, "matmul_reduce_scatter: shape=(%d,%d,%d) dtype=%s rank=%d/%d", M, N, K, A.dtype, rank,
+                 world_size, rank=rank, num_ranks=world_size)
 
     total_tiles = _tile_count(M, N, config)
     if workspace.locks is not None and workspace.locks.numel() < total_tiles:
