@@ -393,13 +393,18 @@ unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels 
 #endif
 
 // Launches for the 32x32 kernel (decode_kernel.h): at most 32 rows, or any output small enough that
-// its 32x32 tiles make at most two rounds of one workgroup per CU.  Such outputs are a handful of
+// it has at most two 32x32 tiles per CU (two workgroups share a CU then).  Such outputs are a handful of
 // 128x128 tiles - 128 x 1024 is eight of them, on eight of 256 CUs - while the small tiles with K split
 // over the waves of a workgroup keep the whole chip busy (fp16, two-shot, eight ranks: 128x1024x4096 41 ->
-// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 14 us; from about 540 tiles on the tiled kernels win).
-bool decode_sized(const FusedParams& p, int cu_count) {
+// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 9 us; from about 540 tiles on the tiled kernels win at short K).
+// With a long K (from 4096 bytes per row) the small tiles stay ahead up to three per CU - a round of two
+// and a round of one - because the tiled kernel's walk over K is the longer chain (fp16, 192x2880x4096:
+// 36.4 -> 29.9 us, 160x4096x4096 38.1 -> 29.5, 96x8192x4096 38.6 -> 33.5; at K = 512 the 64x128 tiles win by 8 %).
+bool decode_sized(const FusedParams& p, int cu_count, int in_dtype) {
   if (p.M <= 32) return true;
-  return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
+  const long long tiles = (long long)cdiv(p.M, 32) * cdiv(p.N, 32);
+  const long long kbytes = (long long)p.K * (in_dtype == IRIS_HIP_FP8_E4M3 ? 1 : 2);
+  return tiles <= 2ll * cu_count || (tiles <= 3ll * cu_count && kbytes >= 4096);
 }
 // ... and whose A that kernel can fetch: not gathered, gathered by rows in whole 32-row tiles per slot, or
 // gathered along K with every wave's 256 bytes of K inside one slot.
@@ -449,7 +454,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
-  else if (decode_sized(p, facts->cu_count) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count, in_dtype) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
   else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
            !(p.gather == GATHER_M && p.M_local % 64))
     kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own
