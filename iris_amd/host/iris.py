@@ -13,6 +13,7 @@ import logging
 import os
 
 import torch
+import torch.distributed as _dist
 
 from . import tensors as tensor_creation
 from .heap import SymmetricHeap
@@ -92,6 +93,9 @@ class Iris:
             self._status = torch.zeros(1, dtype=torch.int32, pin_memory=True)
         else:
             self._status = torch.zeros(1, dtype=torch.int32, device=self.heap.device)
+        # The same word as a numpy view: reading one element of a tensor costs microseconds, and every
+        # synchronous operator call ends with such a read.
+        self._status_view = self._status.numpy() if self._status.device.type == "cpu" else None
         # One GPU standing in for all ranks: when set, the fused operators' preambles mark the other
         # ranks as finished (flags raised, aux zeroed) so that a launch does not wait for them.
         self.stand_in_peers = os.environ.get("IRIS_STAND_IN_PEERS", "0") not in ("", "0")
@@ -144,25 +148,24 @@ class Iris:
         that have HIP kernels here: all_reduce (+ preamble) and reduce_scatter."""
 
         def __init__(self, iris_instance):
+            # (imported here: the collectives import this module's package)
+            from ..ccl.all_reduce import all_reduce, all_reduce_preamble
+            from ..ccl.reduce_scatter import reduce_scatter
+
             self._iris = iris_instance
+            self._all_reduce, self._all_reduce_preamble, self._reduce_scatter = all_reduce, all_reduce_preamble, reduce_scatter
 
         def all_reduce_preamble(self, output_tensor, input_tensor, config=None, workspace=None):
-            from ..ccl.all_reduce import all_reduce_preamble
-
-            return all_reduce_preamble(output_tensor, input_tensor, self._iris, config=config, workspace=workspace)
+            return self._all_reduce_preamble(output_tensor, input_tensor, self._iris, config=config, workspace=workspace)
 
         def all_reduce(self, output_tensor, input_tensor, op=None, group=None, async_op=False, config=None,
                        workspace=None):
-            from ..ccl.all_reduce import all_reduce
-
-            return all_reduce(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
-                              config=config, workspace=workspace)
+            return self._all_reduce(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
+                                    config=config, workspace=workspace)
 
         def reduce_scatter(self, output_tensor, input_tensor, op=None, group=None, async_op=False, config=None):
-            from ..ccl.reduce_scatter import reduce_scatter
-
-            reduce_scatter(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
-                           config=config)
+            self._reduce_scatter(output_tensor, input_tensor, self._iris, op=op, group=group, async_op=async_op,
+                                 config=config)
 
         def __getattr__(self, name):
             if name in ("all_to_all", "all_gather"):
@@ -278,15 +281,13 @@ class Iris:
                 torch.cuda.synchronize()
             else:
                 stream.synchronize()
-        import torch.distributed as dist
-
-        if dist.is_available() and dist.is_initialized():
-            dist.barrier(group=group)
+        if _dist.is_available() and _dist.is_initialized():
+            _dist.barrier(group=group)
         self.check_status()
 
     def check_status(self):
         """Raise RuntimeError if a kernel set a status bit since the last check (needs a sync first)."""
-        status = int(self._status[0])
+        status = int(self._status_view[0]) if self._status_view is not None else int(self._status[0])
         if status:
             self._status.zero_()
             raise RuntimeError(
