@@ -13,7 +13,8 @@
 //     is short), loads exactly
 //     the operand bytes it multiplies (direct-to-LDS, into a region no other wave touches) and waits for
 //     nothing but its own loads - the K phase has no workgroup barrier; problems whose K fits one or two
-//     chunks (K <= 2048 bytes) have every operand load in flight from the first instruction on;
+//     chunks (K <= 2048 bytes with 256-byte shares, 1024 with 128-byte shares) have every operand load in
+//     flight from the first instruction on;
 //   * a fifth wave multiplies nothing.  Its first instructions, issued while the other four waves still
 //     set up their loaders, are probes of the peers' flags (direct-to-LDS, system scope): the oldest loads
 //     of the CU.  That matters because a CU's vector memory pipeline returns in order - a probe issued
