@@ -971,7 +971,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
         // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
         // at a time also with seven peers, and groups below the last row of the matrix are skipped.
-        constexpr int G = (NP >= 4 && NW == 8) ? 2 : 4;
+        constexpr int G0 = (NP >= 4 && NW == 8) ? 2 : 4;
+        constexpr int G = G0 < PASSES ? G0 : PASSES;
         static_assert(PASSES % G == 0, "pass grouping");
         const int npasses = RECT ? cdiv((r1 - r0) * ncw, NT) : PASSES;
         for (int pg = 0; pg < npasses; pg += G) {
@@ -1151,13 +1152,15 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
 //           problems (half the operand bytes per flop of the 128x128 tiles).
 //   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
 //   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
+//   skinny64  64x64, 4 waves of one 32x32 block each, 256-byte K steps, 3-slot ring: outputs of at most one
+//           such tile per CU, which the 64x128 tiles would spread over half the CUs.
 // Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
 // smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
 //   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
 //           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
 //           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
 //           tiles the shorter K steps make it the slower of the two.
-enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4 };
+enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4, TILE_SKINNY64 = 5 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
   return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
 }
@@ -1169,9 +1172,13 @@ template <int IN, bool BKC>
 using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
 template <int IN, bool BKC>
 using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
+template <int IN, bool BKC>
+using Skinny64Tile = MfmaCfg<IN, 64, 64, tile_bk(TILE_SKINNY64, IN), 2, 2, 3, BKC>;
 
-inline int tile_rows(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_SKINNY ? 64 : kind == TILE_DECODE ? 32 : 128; }
-inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_DECODE ? 32 : 128; }
+inline int tile_rows(int kind) {
+  return kind == TILE_BIG ? 256 : (kind == TILE_SKINNY || kind == TILE_SKINNY64) ? 64 : kind == TILE_DECODE ? 32 : 128;
+}
+inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_DECODE ? 32 : kind == TILE_SKINNY64 ? 64 : 128; }
 
 #include "decode_kernel.h"
 
@@ -1219,6 +1226,8 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
       return bkc ? launch_mfma<SmallTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, device, cu, s, name);
     case TILE_SMALL2:
       return bkc ? launch_mfma<Small2Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, device, cu, s, name);
+    case TILE_SKINNY64:
+      return bkc ? launch_mfma<Skinny64Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Skinny64Tile<IN, false>>(p, device, cu, s, name);
     default:
       return bkc ? launch_mfma<SkinnyTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SkinnyTile<IN, false>>(p, device, cu, s, name);
   }
