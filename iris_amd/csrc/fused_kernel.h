@@ -1152,8 +1152,10 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
 //           problems (half the operand bytes per flop of the 128x128 tiles).
 //   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
 //   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
-//   skinny64  64x64, 4 waves of one 32x32 block each, 256-byte K steps, 3-slot ring: outputs of at most one
-//           such tile per CU, which the 64x128 tiles would spread over half the CUs.
+//   skinny64  64x64, 4 waves of one 32x32 block each, 128-byte K steps, 4-slot ring of 64 KiB (two
+//           workgroups per CU): outputs of at most two such tiles per CU, which wider tiles would spread
+//           over a part of the CUs.  (With 256-byte steps and three slots the same tile is 5-15 % slower:
+//           fp16, two-shot, eight ranks, 256x4096x512 12.2 against 11.6 us, 256x4096x4096 33.2 against 27.7.)
 // Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
 // smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
 //   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
@@ -1162,7 +1164,7 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
 //           tiles the shorter K steps make it the slower of the two.
 enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4, TILE_SKINNY64 = 5 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
-  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : kind == TILE_SMALL ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
+  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : (kind == TILE_SMALL || kind == TILE_SKINNY64) ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
 }
 template <int IN, bool BKC>
 using BigTile = MfmaCfg<IN, 256, 256, tile_bk(TILE_BIG, IN), 2, 4, 4, BKC>;
@@ -1173,7 +1175,7 @@ using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
 template <int IN, bool BKC>
 using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
 template <int IN, bool BKC>
-using Skinny64Tile = MfmaCfg<IN, 64, 64, tile_bk(TILE_SKINNY64, IN), 2, 2, 3, BKC>;
+using Skinny64Tile = MfmaCfg<IN, 64, 64, tile_bk(TILE_SKINNY64, IN), 2, 2, 4, BKC>;
 
 inline int tile_rows(int kind) {
   return kind == TILE_BIG ? 256 : (kind == TILE_SKINNY || kind == TILE_SKINNY64) ? 64 : kind == TILE_DECODE ? 32 : 128;

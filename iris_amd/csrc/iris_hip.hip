@@ -449,16 +449,17 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64x128 tiles for M <= 64 and for outputs
   // that are at most one such tile per CU (128x128 tiles would leave half the chip idle: fp16, two-shot,
   // eight ranks, 512x4096x512 21.3 -> 15.7 us, 256x8192x4096 48.5 -> 42.3 us, 1024x2048x512 21.0 -> 15.9 us), else
-  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Outputs of at most one 64x64
-  // tile per CU take those (256x4096x512 14.4 -> 12.0 us, 1024x1024x4096 38.1 -> 31.9 us against 64x128 tiles on
-  // half the CUs; with more than one round of them the wider tiles win: 512x4096x4096 44 against 57 us).
+  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Outputs of at most two 64x64
+  // tiles per CU take those, two workgroups per CU (fp16, two-shot, eight ranks, against 64x128 tiles:
+  // 256x4096x512 14.4 -> 11.6 us, 256x4096x4096 38.3 -> 27.7, 512x4096x512 15.2 -> 13.0, 640x2880x4096 42.5 -> 35.8;
+  // from 630 such tiles on the 128x128 tiles win: 896x2880x4096 46 against 55 us).
   // Small outputs (decode_sized) take the latency-oriented 32x32 kernel (decode_kernel.h).
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
   else if (decode_sized(p, facts->cu_count, in_dtype) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
-  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= facts->cu_count && !(p.gather == GATHER_M && p.M_local % 64))
-    kind = TILE_SKINNY64;  // every 64x64 tile gets a CU of its own: twice the workgroups of the 64x128 tiles
+  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= 2ll * facts->cu_count && !(p.gather == GATHER_M && p.M_local % 64))
+    kind = TILE_SKINNY64;  // all 64x64 tiles resident at once, two workgroups per CU
   else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
            !(p.gather == GATHER_M && p.M_local % 64))
     kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own

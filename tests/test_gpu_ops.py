@@ -664,9 +664,9 @@ def test_ragged_shapes_mfma(M, N, K, variant):
 
 # Tile counts that are not a multiple of the eight XCDs: the launch grid is rounded up and the surplus
 # workgroups must find no tile (90, 180, 270 and 432 tiles of 32x32 - one and two rounds of the small-output
-# kernel -, 132 of 64x64, 129 of 64x128, 184 of 128x128, 140 of 256x256).
+# kernel -, 132 and 405 of 64x64 - one and two workgroups per CU -, 257 of 64x128, 184 of 128x128, 140 of 256x256).
 @pytest.mark.parametrize("M,N,K,tile", [(32, 2880, 64, "32x32"), (48, 2880, 64, "32x32"), (96, 2880, 64, "32x32"),
-                                        (384, 1152, 96, "32x32"), (48, 8400, 64, "64x64"), (48, 16400, 64, "64x128"), (1000, 2880, 64, "128x128"),
+                                        (384, 1152, 96, "32x32"), (48, 8400, 64, "64x64"), (300, 5184, 64, "64x64"), (48, 32848, 64, "64x128"), (1000, 2880, 64, "128x128"),
                                         (2560, 3584, 64, "256x256")])
 def test_tile_counts_off_the_xcd_multiple(M, N, K, tile):
     W, rank, dtype = 2, 1, torch.float16
