@@ -396,15 +396,12 @@ unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels 
 // it has at most two 32x32 tiles per CU (two workgroups share a CU then).  Such outputs are a handful of
 // 128x128 tiles - 128 x 1024 is eight of them, on eight of 256 CUs - while the small tiles with K split
 // over the waves of a workgroup keep the whole chip busy (fp16, two-shot, eight ranks: 128x1024x4096 41 ->
-// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 9 us; from about 540 tiles on the tiled kernels win at short K).
-// With a long K (from 4096 bytes per row) the small tiles stay ahead up to three per CU - a round of two
-// and a round of one - because the tiled kernel's walk over K is the longer chain (fp16, 192x2880x4096:
-// 36.4 -> 29.9 us, 160x4096x4096 38.1 -> 29.5, 96x8192x4096 38.6 -> 33.5; at K = 512 the 64x128 tiles win by 8 %).
-bool decode_sized(const FusedParams& p, int cu_count, int in_dtype) {
+// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 9 us).
+// Beyond two tiles per CU the 64x64 tiled kernel is ahead at every K (fp16, 192x2880x4096: 25.0 against 29.4 us
+// for this kernel in a round of two and a round of one per CU; 640x1024x4096: 26.7 against 35.1).
+bool decode_sized(const FusedParams& p, int cu_count) {
   if (p.M <= 32) return true;
-  const long long tiles = (long long)cdiv(p.M, 32) * cdiv(p.N, 32);
-  const long long kbytes = (long long)p.K * (in_dtype == IRIS_HIP_FP8_E4M3 ? 1 : 2);
-  return tiles <= 2ll * cu_count || (tiles <= 3ll * cu_count && kbytes >= 4096);
+  return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
 }
 // ... and whose A that kernel can fetch: not gathered, gathered by rows in whole 32-row tiles per slot, or
 // gathered along K with every wave's 256 bytes of K inside one slot.
@@ -457,7 +454,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
-  else if (decode_sized(p, facts->cu_count, in_dtype) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
   else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= 2ll * facts->cu_count && !(p.gather == GATHER_M && p.M_local % 64))
     kind = TILE_SKINNY64;  // all 64x64 tiles resident at once, two workgroups per CU
   else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&

@@ -23,7 +23,7 @@ NAMES = {torch.bfloat16: "bf16", torch.float16: "f16", FP8: "fp8"}
 # Shapes that make the host pick each tile shape on a 256-CU part: >= 136 tiles of 256x256 (big), at
 # most 256 tiles of 128x128 but more than 256 of 64x128 (small), more than 256 of 128x128 (small2, two
 # workgroups per CU), M <= 64 or at most 256 tiles of 64x128 (skinny), at most 512 tiles of 64x64;
-# outputs of at most 512 tiles of 32x32 (768 when K is at least 4096 bytes) take the small-output kernel
+# outputs of at most 512 tiles of 32x32 take the small-output kernel
 # (one row tile, six of them, and more tiles than CUs: two workgroups per CU, K in chunks of half the size).
 TILE_SHAPES = {
     "256x256": (3072, 3072, 80),
@@ -34,7 +34,7 @@ TILE_SHAPES = {
     "32x32": (32, 1168, 1360),       # at most 32 rows: K in 1024-byte chunks (2 or 3 here)
     "32x32m": (176, 400, 1360),      # 6 x 13 tiles, the last row tile half empty
     "32x32h": (96, 2768, 1360),      # 3 x 87 tiles: 512-byte chunks, the last one ragged across the waves
-    "32x32t": (192, 2864, 4112),     # 6 x 90 tiles, more than two per CU: taken for long K only
+    "64x64l": (192, 2864, 4112),     # 135 tiles of 64x64 (540 of 32x32: past the small-output kernel), long K
 }
 
 
@@ -57,7 +57,7 @@ def _scales(dtype):
 @pytest.mark.parametrize("tile", sorted(TILE_SHAPES))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, FP8], ids=lambda d: NAMES[d])
 def test_every_build_bit_exact(dtype, tile, layout):
-    """3 input types x 6 kernels (the small-output one at four shapes) x 2 layouts of B through
+    """3 input types x 6 kernels (the small-output one at three shapes, the 64x64 tile at two) x 2 layouts of B through
     matmul_all_reduce with three peers."""
     M, N, K = TILE_SHAPES[tile]
     W, rank = 4, 2
@@ -74,9 +74,9 @@ def test_every_build_bit_exact(dtype, tile, layout):
     stage_peers(ctx, ws, peers)
     ops.matmul_all_reduce(ctx, dC, dA, dB, config=cfg, workspace=ws, kernel_path="mfma", **_scales(dtype))
     kernel = _lib.last_kernel()
-    assert kernel.startswith(f"mfma_{NAMES[dtype]}_{tile[:7].rstrip('sdmht')}") and kernel.endswith("_" + layout), kernel
+    assert kernel.startswith(f"mfma_{NAMES[dtype]}_{tile[:7].rstrip('sdmhl')}") and kernel.endswith("_" + layout), kernel
     kstep = int(kernel.split("x")[2].split("_")[0]) * (1 if dtype == FP8 else 2)  # bytes per K step
-    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 256, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "32x32t": 512}[tile], kernel
+    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 256, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "64x64l": 128}[tile], kernel
     scale = 0.5 if dtype == FP8 else 1.0
     exp = oracle.matmul_all_reduce(A, B, peers, rank, W, bm, 64, variant, out_dtype=out_dtype, scale=scale)
     assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"{kernel}: aux")
