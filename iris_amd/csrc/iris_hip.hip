@@ -460,8 +460,11 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
            !(p.gather == GATHER_M && p.M_local % 64))
     kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own
+  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= 2ll * facts->cu_count && (long long)p.K * elem_size(in_dtype) <= 2048 &&
+           !(p.gather == GATHER_M && p.M_local % 64))
+    kind = TILE_SKINNYD;  // short K: 64x128 tiles, two workgroups per CU (see the tile list in fused_kernel.h)
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
-  // IRIS_HIP_TILE = big | small | small2 | skinny | skinny64 overrides the choice among the tiled kernels (a tuning
+  // IRIS_HIP_TILE = big | small | small2 | skinny | skinnyd | skinny64 overrides the choice among the tiled kernels (a tuning
   // aid; results do not depend on the tile shape beyond the order of the fp32 sums over K).
   static const int forced_tile = [] {
     const char* e = getenv("IRIS_HIP_TILE");
@@ -471,6 +474,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     if (!strcmp(e, "small2")) return (int)TILE_SMALL2;
     if (!strcmp(e, "skinny")) return (int)TILE_SKINNY;
     if (!strcmp(e, "skinny64")) return (int)TILE_SKINNY64;
+    if (!strcmp(e, "skinnyd")) return (int)TILE_SKINNYD;
     return -1;
   }();
   if (forced_tile >= 0 && kind != TILE_DECODE &&

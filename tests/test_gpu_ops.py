@@ -589,8 +589,8 @@ def test_c_abi_rejects_bad_arguments():
 # ------------------------------------------------------------------------------------------------
 # HIP graphs: a launch is one kernel node, so launch-bound loops can be captured and replayed
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("M,N,K,kernel", [(1280, 3072, 160, "128x128"), (256, 384, 160, "32x32"), (32, 1168, 1360, "32x32"),
-                                          (3072, 3072, 80, "256x256")])
+@pytest.mark.parametrize("M,N,K,kernel", [(1280, 3072, 1040, "128x128"), (1280, 3072, 160, "64x128"), (256, 384, 160, "32x32"),
+                                          (32, 1168, 1360, "32x32"), (3072, 3072, 80, "256x256")])
 @pytest.mark.parametrize("variant", ["one_shot", "two_shot"])
 def test_graph_replay_matches_eager(variant, M, N, K, kernel):
     """Captured once, replayed four times with new operands: the tiled kernels and the small-output kernel
@@ -664,9 +664,10 @@ def test_ragged_shapes_mfma(M, N, K, variant):
 
 # Tile counts that are not a multiple of the eight XCDs: the launch grid is rounded up and the surplus
 # workgroups must find no tile (90, 180, 270 and 432 tiles of 32x32 - one and two rounds of the small-output
-# kernel -, 132 and 405 of 64x64 - one and two workgroups per CU -, 257 of 64x128, 184 of 128x128, 140 of 256x256).
+# kernel -, 132 and 405 of 64x64 - one and two workgroups per CU -, 257 and 368 of 64x128 - the same -, 184 of
+# 128x128, 140 of 256x256).
 @pytest.mark.parametrize("M,N,K,tile", [(32, 2880, 64, "32x32"), (48, 2880, 64, "32x32"), (96, 2880, 64, "32x32"),
-                                        (384, 1152, 96, "32x32"), (48, 8400, 64, "64x64"), (300, 5184, 64, "64x64"), (48, 32848, 64, "64x128"), (1000, 2880, 64, "128x128"),
+                                        (384, 1152, 96, "32x32"), (48, 8400, 64, "64x64"), (300, 5184, 64, "64x64"), (48, 32848, 64, "64x128"), (1000, 2880, 64, "64x128"), (1000, 2880, 1032, "128x128"),
                                         (2560, 3584, 64, "256x256")])
 def test_tile_counts_off_the_xcd_multiple(M, N, K, tile):
     W, rank, dtype = 2, 1, torch.float16

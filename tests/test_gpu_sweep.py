@@ -27,7 +27,8 @@ NAMES = {torch.bfloat16: "bf16", torch.float16: "f16", FP8: "fp8"}
 # (one row tile, six of them, and more tiles than CUs: two workgroups per CU, K in chunks of half the size).
 TILE_SHAPES = {
     "256x256": (3072, 3072, 80),
-    "128x128s": (1280, 3072, 208),   # 128-byte K steps
+    "128x128s": (1280, 3072, 2064),  # 128-byte K steps
+    "64x128d": (1280, 3072, 208),    # 480 tiles of 64x128 and a short K: two workgroups per CU, 128-byte K steps
     "128x128d": (2304, 2048, 80),    # 64-byte K steps, two workgroups per CU
     "64x128": (48, 32832, 336),      # 513 tiles of 64x64, 257 of 64x128
     "64x64": (48, 8320, 336),        # 130 tiles of 64x64
@@ -57,7 +58,7 @@ def _scales(dtype):
 @pytest.mark.parametrize("tile", sorted(TILE_SHAPES))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, FP8], ids=lambda d: NAMES[d])
 def test_every_build_bit_exact(dtype, tile, layout):
-    """3 input types x 6 kernels (the small-output one at three shapes, the 64x64 tile at two) x 2 layouts of B through
+    """3 input types x 7 kernels (the small-output one at three shapes, the 64x64 tile at two) x 2 layouts of B through
     matmul_all_reduce with three peers."""
     M, N, K = TILE_SHAPES[tile]
     W, rank = 4, 2
@@ -76,7 +77,7 @@ def test_every_build_bit_exact(dtype, tile, layout):
     kernel = _lib.last_kernel()
     assert kernel.startswith(f"mfma_{NAMES[dtype]}_{tile[:7].rstrip('sdmhl')}") and kernel.endswith("_" + layout), kernel
     kstep = int(kernel.split("x")[2].split("_")[0]) * (1 if dtype == FP8 else 2)  # bytes per K step
-    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 256, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "64x64l": 128}[tile], kernel
+    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 256, "64x128d": 128, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "64x64l": 128}[tile], kernel
     scale = 0.5 if dtype == FP8 else 1.0
     exp = oracle.matmul_all_reduce(A, B, peers, rank, W, bm, 64, variant, out_dtype=out_dtype, scale=scale)
     assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"{kernel}: aux")
