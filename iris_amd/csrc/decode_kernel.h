@@ -1,4 +1,4 @@
-// Small outputs - decode-sized launches (M <= 32 rows) and, more generally, outputs of at most two
+// Small outputs - decode-sized launches (a few rows) and, more generally, outputs of at most two
 // 32 x 32 tiles per CU - of every operator: fused_decode_kernel.  The description
 // follows the flag-carrying operators; the others leave after the partial tiles have met.
 //

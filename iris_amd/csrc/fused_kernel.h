@@ -1151,24 +1151,26 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
 //   big     256x256, 8 waves, 4-slot ring: 128 accumulator registers per lane, the shape for large
 //           problems (half the operand bytes per flop of the 128x128 tiles).
 //   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
-//   skinny  64x128, 4 waves, 256-byte K steps, 3-slot ring: decode-sized M (<= 64 rows).
-//   skinnyd 64x128, 4 waves, 128-byte K steps, 3-slot ring of 72 KiB (two workgroups per CU): outputs of
-//           257-512 such tiles with a short K (at most 2048 bytes per row), where it is 8-13 % ahead of the
-//           128x128 tiles (896x2880x512 18.6 -> 16.5 us, 1024x4096x512 23.9 -> 21.9); at K = 1376 the two tie,
-//           at K = 4096 it is 10-20 % behind.
-//   skinny64  64x64, 4 waves of one 32x32 block each, 128-byte K steps, 4-slot ring of 64 KiB (two
-//           workgroups per CU): outputs of at most two such tiles per CU, which wider tiles would spread
-//           over a part of the CUs.  (With 256-byte steps and three slots the same tile is 5-15 % slower:
-//           fp16, two-shot, eight ranks, 256x4096x512 12.2 against 11.6 us, 256x4096x4096 33.2 against 27.7.)
-// Short problems pay a fixed latency per K step (barrier, LDS round trip, dependent MFMAs), so the
-// smaller tiles take fewer, fatter steps and keep as many bytes in flight as LDS allows.
 //   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
 //           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
 //           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
 //           tiles the shorter K steps make it the slower of the two.
-enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4, TILE_SKINNY64 = 5, TILE_SKINNYD = 6 };
+//   skinny  64x128, 4 waves, 128-byte K steps, 3-slot ring of 72 KiB: two workgroups per CU.  Outputs of at
+//           most 64 rows that are too wide for the kernels below (fp16, two-shot, eight ranks, against the
+//           256x256 tile that the tile count alone would pick: 32x40960x2048 51 -> 38 us, 64x131072x2048
+//           150 -> 130 us), and outputs of 257-512 such tiles with a short K (at most 2048 bytes per row),
+//           where it is 8-13 % ahead of the 128x128 tiles (896x2880x512 18.6 -> 16.5 us, 1024x4096x512
+//           23.9 -> 21.9); at K = 1376 the two tie, at K = 4096 it is 10-20 % behind.  (With 256-byte steps
+//           and one workgroup per CU the same tile was 25-45 % slower on the wide outputs.)
+//   skinny64  64x64, 4 waves of one 32x32 block each, 128-byte K steps, 4-slot ring of 64 KiB (two
+//           workgroups per CU): outputs of at most two such tiles per CU, which wider tiles would spread
+//           over a part of the CUs.  (With 256-byte steps and three slots the same tile is 5-15 % slower:
+//           fp16, two-shot, eight ranks, 256x4096x512 12.2 against 11.6 us, 256x4096x4096 33.2 against 27.7.)
+// The small tiles keep as many bytes in flight as LDS allows; what pays is residency - every tile of the
+// output on a CU at the same time - before fat K steps.
+enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4, TILE_SKINNY64 = 5 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
-  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : (kind == TILE_SMALL || kind == TILE_SKINNY64 || kind == TILE_SKINNYD) ? 128 : 256) / (in == IN_FP8 ? 1 : 2);
+  return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : 128) / (in == IN_FP8 ? 1 : 2);
 }
 template <int IN, bool BKC>
 using BigTile = MfmaCfg<IN, 256, 256, tile_bk(TILE_BIG, IN), 2, 4, 4, BKC>;
@@ -1179,12 +1181,10 @@ using SkinnyTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNY, IN), 2, 2, 3, BKC>;
 template <int IN, bool BKC>
 using Small2Tile = MfmaCfg<IN, 128, 128, tile_bk(TILE_SMALL2, IN), 2, 2, 4, BKC>;
 template <int IN, bool BKC>
-using SkinnyDTile = MfmaCfg<IN, 64, 128, tile_bk(TILE_SKINNYD, IN), 2, 2, 3, BKC>;
-template <int IN, bool BKC>
 using Skinny64Tile = MfmaCfg<IN, 64, 64, tile_bk(TILE_SKINNY64, IN), 2, 2, 4, BKC>;
 
 inline int tile_rows(int kind) {
-  return kind == TILE_BIG ? 256 : (kind == TILE_SKINNY || kind == TILE_SKINNY64 || kind == TILE_SKINNYD) ? 64 : kind == TILE_DECODE ? 32 : 128;
+  return kind == TILE_BIG ? 256 : (kind == TILE_SKINNY || kind == TILE_SKINNY64) ? 64 : kind == TILE_DECODE ? 32 : 128;
 }
 inline int tile_cols(int kind) { return kind == TILE_BIG ? 256 : kind == TILE_DECODE ? 32 : kind == TILE_SKINNY64 ? 64 : 128; }
 
@@ -1234,8 +1234,6 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
       return bkc ? launch_mfma<SmallTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SmallTile<IN, false>>(p, device, cu, s, name);
     case TILE_SMALL2:
       return bkc ? launch_mfma<Small2Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Small2Tile<IN, false>>(p, device, cu, s, name);
-    case TILE_SKINNYD:
-      return bkc ? launch_mfma<SkinnyDTile<IN, true>>(p, device, cu, s, name) : launch_mfma<SkinnyDTile<IN, false>>(p, device, cu, s, name);
     case TILE_SKINNY64:
       return bkc ? launch_mfma<Skinny64Tile<IN, true>>(p, device, cu, s, name) : launch_mfma<Skinny64Tile<IN, false>>(p, device, cu, s, name);
     default:

@@ -392,15 +392,16 @@ void heap_bases_from_registry(FusedParams& p, const int64_t* context_tensor) {
 unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
 #endif
 
-// Launches for the 32x32 kernel (decode_kernel.h): at most 32 rows, or any output small enough that
-// it has at most two 32x32 tiles per CU (two workgroups share a CU then).  Such outputs are a handful of
+// Launches for the 32x32 kernel (decode_kernel.h): any output small enough that it has at most two 32x32
+// tiles per CU (two workgroups share a CU then) - decode-sized launches of up to 32 x 16384, and taller
+// ones of the same area.  Such outputs are a handful of
 // 128x128 tiles - 128 x 1024 is eight of them, on eight of 256 CUs - while the small tiles with K split
 // over the waves of a workgroup keep the whole chip busy (fp16, two-shot, eight ranks: 128x1024x4096 41 ->
 // 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 9 us).
 // Beyond two tiles per CU the 64x64 tiled kernel is ahead at every K (fp16, 192x2880x4096: 25.0 against 29.4 us
-// for this kernel in a round of two and a round of one per CU; 640x1024x4096: 26.7 against 35.1).
+// for this kernel in a round of two and a round of one per CU; 640x1024x4096: 26.7 against 35.1; 32x32768x4096:
+// 51 against 66).
 bool decode_sized(const FusedParams& p, int cu_count) {
-  if (p.M <= 32) return true;
   return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
 }
 // ... and whose A that kernel can fetch: not gathered, gathered by rows in whole 32-row tiles per slot, or
@@ -442,29 +443,22 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   p.num_xcd = facts->xcc_count;
   hipStream_t s = (hipStream_t)stream;
 
-  // Tile choice: the 256x256 tile from about half the CUs busy (measured cross-over against the
-  // 128x128 tiles: between 128 and 144 big tiles on 256 CUs), 64x128 tiles for M <= 64 and for outputs
-  // that are at most one such tile per CU (128x128 tiles would leave half the chip idle: fp16, two-shot,
-  // eight ranks, 512x4096x512 21.3 -> 15.7 us, 256x8192x4096 48.5 -> 42.3 us, 1024x2048x512 21.0 -> 15.9 us), else
-  // 128x128 - two workgroups per CU when there are more such tiles than CUs.  Outputs of at most two 64x64
-  // tiles per CU take those, two workgroups per CU (fp16, two-shot, eight ranks, against 64x128 tiles:
-  // 256x4096x512 14.4 -> 11.6 us, 256x4096x4096 38.3 -> 27.7, 512x4096x512 15.2 -> 13.0, 640x2880x4096 42.5 -> 35.8;
-  // from 630 such tiles on the 128x128 tiles win: 896x2880x4096 46 against 55 us).
-  // Small outputs (decode_sized) take the latency-oriented 32x32 kernel (decode_kernel.h).
+  // Tile choice (the tile list in fused_kernel.h has the measurements): the 256x256 tile from about half the
+  // CUs busy (cross-over against the 128x128 tiles between 128 and 144 big tiles on 256 CUs) unless the output
+  // has at most 64 rows; the latency-oriented 32x32 kernel (decode_kernel.h) for at most two such tiles per CU;
+  // 64x64 tiles for at most two of those per CU; 64x128 tiles for at most 64 rows, and for at most two such
+  // tiles per CU when K is short; else 128x128 - two workgroups per CU when there are more such tiles than CUs.
   const long long big_tiles = (long long)cdiv(p.M, 256) * cdiv(p.N, 256);
+  const bool rows64_ok = !(p.gather == GATHER_M && p.M_local % 64);
   int kind = TILE_SMALL;
-  if (big_tiles * 100 >= (long long)facts->cu_count * 53) kind = TILE_BIG;
+  if (big_tiles * 100 >= (long long)facts->cu_count * 53 && !(p.M <= 64 && rows64_ok)) kind = TILE_BIG;
   else if (decode_sized(p, facts->cu_count) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
-  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= 2ll * facts->cu_count && !(p.gather == GATHER_M && p.M_local % 64))
-    kind = TILE_SKINNY64;  // all 64x64 tiles resident at once, two workgroups per CU
-  else if ((p.M <= 64 || (long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= facts->cu_count) &&
-           !(p.gather == GATHER_M && p.M_local % 64))
-    kind = TILE_SKINNY;  // 64-row tiles also for taller outputs, as long as every 64x128 tile gets a CU of its own
-  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= 2ll * facts->cu_count && (long long)p.K * elem_size(in_dtype) <= 2048 &&
-           !(p.gather == GATHER_M && p.M_local % 64))
-    kind = TILE_SKINNYD;  // short K: 64x128 tiles, two workgroups per CU (see the tile list in fused_kernel.h)
+  else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= 2ll * facts->cu_count && rows64_ok) kind = TILE_SKINNY64;
+  else if (rows64_ok && (p.M <= 64 || ((long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= 2ll * facts->cu_count &&
+                                       (long long)p.K * elem_size(in_dtype) <= 2048)))
+    kind = TILE_SKINNY;
   else if ((long long)cdiv(p.M, 128) * cdiv(p.N, 128) > facts->cu_count) kind = TILE_SMALL2;
-  // IRIS_HIP_TILE = big | small | small2 | skinny | skinnyd | skinny64 overrides the choice among the tiled kernels (a tuning
+  // IRIS_HIP_TILE = big | small | small2 | skinny | skinny64 overrides the choice among the tiled kernels (a tuning
   // aid; results do not depend on the tile shape beyond the order of the fp32 sums over K).
   static const int forced_tile = [] {
     const char* e = getenv("IRIS_HIP_TILE");
@@ -474,7 +468,6 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     if (!strcmp(e, "small2")) return (int)TILE_SMALL2;
     if (!strcmp(e, "skinny")) return (int)TILE_SKINNY;
     if (!strcmp(e, "skinny64")) return (int)TILE_SKINNY64;
-    if (!strcmp(e, "skinnyd")) return (int)TILE_SKINNYD;
     return -1;
   }();
   if (forced_tile >= 0 && kind != TILE_DECODE &&

@@ -22,15 +22,15 @@ NAMES = {torch.bfloat16: "bf16", torch.float16: "f16", FP8: "fp8"}
 
 # Shapes that make the host pick each tile shape on a 256-CU part: >= 136 tiles of 256x256 (big), at
 # most 256 tiles of 128x128 but more than 256 of 64x128 (small), more than 256 of 128x128 (small2, two
-# workgroups per CU), M <= 64 or at most 256 tiles of 64x128 (skinny), at most 512 tiles of 64x64;
+# workgroups per CU), M <= 64 or at most 512 tiles of 64x128 with a short K (skinny), at most 512 tiles of 64x64;
 # outputs of at most 512 tiles of 32x32 take the small-output kernel
 # (one row tile, six of them, and more tiles than CUs: two workgroups per CU, K in chunks of half the size).
 TILE_SHAPES = {
     "256x256": (3072, 3072, 80),
     "128x128s": (1280, 3072, 2064),  # 128-byte K steps
-    "64x128d": (1280, 3072, 208),    # 480 tiles of 64x128 and a short K: two workgroups per CU, 128-byte K steps
+    "64x128m": (1280, 3072, 208),    # 480 tiles of 64x128 and a short K
     "128x128d": (2304, 2048, 80),    # 64-byte K steps, two workgroups per CU
-    "64x128": (48, 32832, 336),      # 513 tiles of 64x64, 257 of 64x128
+    "64x128": (48, 32832, 336),      # at most 64 rows: 513 tiles of 64x64, 257 of 64x128
     "64x64": (48, 8320, 336),        # 130 tiles of 64x64
     "32x32": (32, 1168, 1360),       # at most 32 rows: K in 1024-byte chunks (2 or 3 here)
     "32x32m": (176, 400, 1360),      # 6 x 13 tiles, the last row tile half empty
@@ -77,7 +77,7 @@ def test_every_build_bit_exact(dtype, tile, layout):
     kernel = _lib.last_kernel()
     assert kernel.startswith(f"mfma_{NAMES[dtype]}_{tile[:7].rstrip('sdmhl')}") and kernel.endswith("_" + layout), kernel
     kstep = int(kernel.split("x")[2].split("_")[0]) * (1 if dtype == FP8 else 2)  # bytes per K step
-    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 256, "64x128d": 128, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "64x64l": 128}[tile], kernel
+    assert kstep == {"256x256": 64, "128x128s": 128, "128x128d": 64, "64x128": 128, "64x128m": 128, "64x64": 128, "32x32": 1024, "32x32m": 1024, "32x32h": 512, "64x64l": 128}[tile], kernel
     scale = 0.5 if dtype == FP8 else 1.0
     exp = oracle.matmul_all_reduce(A, B, peers, rank, W, bm, 64, variant, out_dtype=out_dtype, scale=scale)
     assert_bits_equal(ws.aux_buffer.cpu(), exp["aux"], f"{kernel}: aux")
