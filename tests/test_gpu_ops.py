@@ -179,7 +179,7 @@ def test_ragged_shapes_generic(M, N, K):
 @pytest.mark.parametrize("M,N,K", [(256, 384, 128), (3072, 3072, 200)])
 def test_transposed_b_and_strided_views(M, N, K):
     """B handed over as the transpose of an (N, K) tensor (K-contiguous) takes the MFMA path too
-    (128x128 tiles for the first shape, 256x256 for the second)."""
+    (the small-output kernel for the first shape, 256x256 tiles for the second)."""
     ctx = _ctx(1, heap=1 << 27)
     dtype = torch.bfloat16
     A, Bt = randint_cpu((M, K), 8, dtype), randint_cpu((N, K), 9, dtype)
@@ -474,12 +474,14 @@ def test_unstaged_peer_flags_time_out():
 
 
 @pytest.mark.parametrize("M,N,K,variant", [(512, 384, 96, "one_shot"), (512, 384, 96, "two_shot"),
-                                           (32, 1168, 1360, "one_shot"), (3072, 3072, 80, "two_shot")])
+                                           (32, 1168, 1360, "one_shot"), (1280, 3072, 1040, "two_shot"),
+                                           (640, 1024, 96, "one_shot"), (3072, 3072, 80, "two_shot")])
 def test_peer_flags_raised_while_the_kernel_waits(M, N, K, variant):
     """The normal case between real ranks: the peers' flags are not up yet when the kernel looks.  The
     launch goes out with the peers' flags at zero; another stream raises them a little later.  The
     kernel must have raised its own flags first, poll (bounded), and then sum what the peers
-    published - on the 128x128, the decode and the 256x256 kernel."""
+    published - on the small-output kernel (several row tiles, and one), the 128x128, the 64x64 and the
+    256x256 kernel."""
     W, rank, dtype = 4, 2, torch.bfloat16
     ctx = _ctx(W, rank)
     A, B = randint_cpu((M, K), 30, dtype), randint_cpu((K, N), 31, dtype)
@@ -494,13 +496,17 @@ def test_peer_flags_raised_while_the_kernel_waits(M, N, K, variant):
             ctx.peer_view(ws.aux_buffer, r).copy_(peers[r])
             ctx.peer_view(ws.locks, r).zero_()
     torch.cuda.synchronize()
-    side = torch.cuda.Stream()
+    # Streams share a few hardware queues, and work behind the polling kernel in its own queue would only
+    # run once the kernel has given up: the flags are raised from four streams, which covers every queue
+    # (raising them twice is harmless).
+    sides = [torch.cuda.Stream() for _ in range(4)]
     ops.matmul_all_reduce(ctx, dC, dA, dB, async_op=True, config=cfg, workspace=ws)
-    with torch.cuda.stream(side):
-        torch.cuda._sleep(2_000_000)  # the launch above is polling by now
-        for r in range(W):
-            if r != rank:
-                ctx.peer_view(ws.locks, r).fill_(1)
+    for side in sides:
+        with torch.cuda.stream(side):
+            torch.cuda._sleep(2_000_000)  # the launch above is polling by now
+            for r in range(W):
+                if r != rank:
+                    ctx.peer_view(ws.locks, r).fill_(1)
     torch.cuda.synchronize()
     ctx.check_status()  # no spin time-out
     exp = oracle.matmul_all_reduce(A, B, peers, rank, W, fbm, 64, variant, "fp32")
@@ -512,12 +518,13 @@ def test_peer_flags_raised_while_the_kernel_waits(M, N, K, variant):
 
 
 @pytest.mark.parametrize("M,N,K,variant", [(512, 384, 96, "one_shot"), (512, 384, 96, "two_shot"),
-                                           (32, 1168, 1360, "one_shot"), (3072, 3072, 80, "one_shot")])
+                                           (32, 1168, 1360, "one_shot"), (1280, 3072, 1040, "two_shot"),
+                                           (640, 1024, 96, "one_shot"), (3072, 3072, 80, "one_shot")])
 def test_unregistered_context_tensor_gives_the_same_bits(M, N, K, variant):
     """The kernels take the heap bases as kernel arguments when the host has registered the context
     tensor's contents, and load them from the tensor otherwise (a binding that never registers).
-    Both routes must produce the same aux, flags and C; the sizes cover the 128x128, 32x32 (decode)
-    and 256x256 kernels."""
+    Both routes must produce the same aux, flags and C; the sizes cover the small-output kernel and the
+    128x128, 64x64 and 256x256 tiles."""
     W, rank, dtype = 4, 1, torch.bfloat16
     A, B = randint_cpu((M, K), 20, dtype), randint_cpu((K, N), 21, dtype)
     peers = [randn_cpu((M, N), 200 + r, dtype) for r in range(W)]
