@@ -65,7 +65,6 @@ class Workload:
 
     name = ""
     dtype = "bf16"
-    bound = "hbm"
 
     def setup(self, iris, world):
         raise NotImplementedError
@@ -156,7 +155,6 @@ class MatmulAllReduce(Workload):
 
 
 class AllGatherMatmul(Workload):
-    bound = "bf16"
 
     def __init__(self, name, M, N, K, b_transposed=False):
         self.name, self.M, self.N, self.K = name, M, N, K
@@ -205,7 +203,6 @@ class MatmulReduceScatter(Workload):
     peers contribute nothing).  accumulate=True: the reference semantics for rank 0 - seven staged peer
     aux buffers, the rank's own row block summed over the slots in fp32 and stored to its C."""
 
-    bound = "bf16"
 
     def __init__(self, name, M, N, K, accumulate=False):
         self.name, self.M, self.N, self.K, self.accumulate = name, M, N, K, accumulate
@@ -271,7 +268,6 @@ class CopyCalibration(Workload):
     """A plain device-to-device copy of known size: what the HBM byte counters read for it scales the
     counters of the real kernels (profiles/ states the factors)."""
 
-    bound = "hbm"
     dtype = "u8"
 
     def __init__(self, name, nbytes):
@@ -301,7 +297,6 @@ class CclCollective(Workload):
     value is reported in TFLOP/s like every other line (one fp32 add per input element), the roofline
     in GB/s of the bytes the launch has to move."""
 
-    bound = "hbm"
 
     def __init__(self, name, op, variant, M, N):
         self.name, self.op, self.variant, self.M, self.N = name, op, variant, M, N
@@ -374,6 +369,17 @@ for _m in (1024, 4096, 16384):
     WORKLOADS[f"matmul_all_reduce_fp16_{_m}x3584x8192"] = (
         lambda m=_m: MatmulAllReduce(f"matmul_all_reduce_fp16_{m}x3584x8192", m, 3584, 8192, fp16=True, variant="two_shot"))
 DEFAULT = "matmul_all_reduce_bf16_4096x4096x1376"
+
+
+def bounding_roof(wl, world):
+    """"hbm" or "mfma": whichever roof takes longer for this workload at this world size - the
+    algorithmic bytes at the HBM peak or the flops at the MFMA peak of the input type.  Workloads without
+    matrix products (copies, stand-alone collectives) are HBM-bound."""
+    if not getattr(wl, "flops", 0) or wl.dtype not in PEAK:
+        return "hbm"
+    t_hbm = wl.algorithmic_bytes(world) / (PEAK["hbm"][0] * 1e9)
+    t_mfma = wl.flops / (PEAK[wl.dtype][0] * 1e12)
+    return "hbm" if t_hbm >= t_mfma else "mfma"
 
 
 def measured_traffic(workload, world):
@@ -524,17 +530,22 @@ def main():
         tflops = wl.flops / (launch_ms * 1e-3) / 1e12
 
     bytes_alg = wl.algorithmic_bytes(args.world)
-    if wl.bound == "hbm":
+    bound = bounding_roof(wl, args.world)
+    if bound == "hbm":
         peak, unit = PEAK["hbm"]
-        achieved = bytes_alg / (launch_ms * 1e-3) / 1e9
+        per_ms = bytes_alg / 1e6  # achieved = per_ms / launch_ms, in GB/s
     else:
         peak, unit = PEAK[wl.dtype]
-        achieved = wl.flops / (launch_ms * 1e-3) / 1e12
-    per_ms = bytes_alg / 1e6 if wl.bound == "hbm" else wl.flops / 1e9  # achieved = per_ms / launch_ms, in GB/s or TFLOP/s
-    roofline = {"bound": "hbm" if wl.bound == "hbm" else "mfma", "achieved": round(achieved, 2), "peak": peak,
+        per_ms = wl.flops / 1e9   # ... or in TFLOP/s
+    achieved = per_ms / launch_ms
+    frac_reference = round(per_ms / statistics.mean(flushed) / peak, 4) if flushed is not None else None
+    roofline = {"bound": bound, "achieved": round(achieved, 2), "peak": peak,
                 "unit": unit, "frac": round(achieved / peak, 4), "traffic": measured_traffic(args.workload, args.world),
                 "kernel": kernel, "flushed": flushed is not None, "priced_on": priced_on,
-                "frac_do_bench": round(per_ms / statistics.mean(flushed) / peak, 4) if flushed is not None else None,
+                # the same fraction under the reference's literal do_bench sequence (host launch path inside the event pair)
+                "frac_reference_protocol": frac_reference, "frac_do_bench": frac_reference,
+                "roof_us": {"hbm": round(bytes_alg / PEAK["hbm"][0] / 1e3, 2),
+                            "mfma": round(wl.flops / PEAK[wl.dtype][0] / 1e6, 2) if wl.dtype in PEAK else None},
                 "launch_ms_mean": round(launch_ms, 5), "launch_ms_median": round(statistics.median(priced), 5),
                 "launch_ms_flushed": _stats(flushed), "launch_ms_flushed_queued": _stats(queued),
                 "launch_ms_back_to_back": _stats(b2b),

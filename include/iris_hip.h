@@ -119,8 +119,12 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The aux buffer, the tile flags and the
  * one-rank context the kernels need live in a static device array of the library
  * (IRIS_HIP_NOALLOC_MAX_AUX_BYTES + 64 KiB + 256 bytes on every GPU the library runs on, held until the
- * process ends).  The call launches a small kernel that clears the flags it is going to use and then the
- * same kernels as iris_hip_matmul_all_reduce; it calls no hipMalloc / hipFree.
+ * process ends).  The call runs every argument check first (a rejected call enqueues nothing), then
+ * launches a small kernel that clears the flags it is going to use and then the same kernels as
+ * iris_hip_matmul_all_reduce; it calls no hipMalloc / hipFree.  On first use per device the library looks up
+ * the array's address (hipGetSymbolAddress) and, per kernel build, sets the kernel's dynamic-LDS attribute:
+ * before capturing calls into a HIP graph, call iris_hip_query() for the device and make one eager call of
+ * each shape class that will be captured, so that nothing but kernel launches happens under capture.
  *
  * Limits (hipErrorInvalidValue with a message otherwise): the bytes aux spans with C's strides,
  * ((M-1)*stride_cm + (N-1)*stride_cn + 1) * sizeof(out element), at most IRIS_HIP_NOALLOC_MAX_AUX_BYTES;

@@ -51,7 +51,7 @@ def main():
         sys.exit("the kernel library was loaded before the diagnostic build could be selected")
     _lib.LIBRARY_PATH = STAMPS_LIB  # the library is loaded on first use
     lib = _lib.library()
-    lib.iris_hip_debug_set_stamps.argtypes = [ctypes.c_void_p]
+    lib.iris_hip_debug_set_stamps.argtypes = [ctypes.c_void_p, ctypes.c_longlong]
     lib.iris_hip_debug_set_stamps.restype = None
     rate_khz = ctypes.c_int(0)
     hip.gpu_try(hip.runtime().hipDeviceGetAttribute(ctypes.byref(rate_khz), 10017, 0))  # hipDeviceAttributeWallClockRate
@@ -73,10 +73,10 @@ def main():
             cache.sum()
         stamps.zero_()
         torch.cuda.synchronize()
-        lib.iris_hip_debug_set_stamps(ctypes.c_void_p(stamps.data_ptr()))
+        lib.iris_hip_debug_set_stamps(ctypes.c_void_p(stamps.data_ptr()), stamps.shape[0])
         wl.step()
         torch.cuda.synchronize()
-        lib.iris_hip_debug_set_stamps(ctypes.c_void_p(0))
+        lib.iris_hip_debug_set_stamps(ctypes.c_void_p(0), 0)
         if rep < 0:
             continue
         t = stamps.cpu()

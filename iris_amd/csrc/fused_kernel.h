@@ -69,7 +69,8 @@ struct FusedParams {
   long long hb_arg[8];
   int hb_in_args;
 #ifdef IRIS_HIP_PHASE_STAMPS
-  unsigned long long* stamps;  // diagnostic build: 16 time stamps per workgroup (see PHASE_STAMP)
+  unsigned long long* stamps;  // diagnostic build: rows of 16 time stamps (see PHASE_STAMP)
+  long long stamp_rows;        // rows the buffer holds; rows beyond it are not written
 #endif
 };
 
@@ -82,7 +83,8 @@ struct FusedParams {
 #ifdef IRIS_HIP_PHASE_STAMPS
 #define PHASE_STAMP(i)                                                                         \
   do {                                                                                         \
-    if (p.stamps && threadIdx.x == 0 && it < 8) p.stamps[(it * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64(); \
+    if (p.stamps && threadIdx.x == 0 && it < 8 && (long long)it * gridDim.x + blockIdx.x < p.stamp_rows)     \
+      p.stamps[((long long)it * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64();                       \
   } while (0)
 #else
 #define PHASE_STAMP(i) \
@@ -357,7 +359,7 @@ __device__ __forceinline__ FusedParams pin_kernel_arguments(const FusedParams& a
   asm volatile("" : "+s"(q.hb_arg[0]), "+s"(q.hb_arg[1]), "+s"(q.hb_arg[2]), "+s"(q.hb_arg[3]), "+s"(q.hb_arg[4]),
                "+s"(q.hb_arg[5]), "+s"(q.hb_arg[6]), "+s"(q.hb_arg[7]));
 #ifdef IRIS_HIP_PHASE_STAMPS
-  asm volatile("" : "+s"(q.stamps));
+  asm volatile("" : "+s"(q.stamps), "+s"(q.stamp_rows));
 #endif
   return q;
 }

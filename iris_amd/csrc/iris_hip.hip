@@ -295,6 +295,17 @@ int launch_generic(FusedParams p, int cu_count, hipStream_t stream, const char* 
   return (int)hipGetLastError();
 }
 
+// Type pairs the generic kernel is built for (the list of dispatch_generic below).
+bool generic_supported(int in_dtype, int out_dtype) {
+  switch (in_dtype) {
+    case IRIS_HIP_BF16: return out_dtype == IRIS_HIP_BF16 || out_dtype == IRIS_HIP_FP32;
+    case IRIS_HIP_FP16: return out_dtype == IRIS_HIP_FP16 || out_dtype == IRIS_HIP_FP32;
+    case IRIS_HIP_FP32: return out_dtype == IRIS_HIP_FP32;
+    case IRIS_HIP_FP8_E4M3: return out_dtype == IRIS_HIP_BF16 || out_dtype == IRIS_HIP_FP16;
+  }
+  return false;
+}
+
 int dispatch_generic(const FusedParams& p, int in_dtype, int out_dtype, int cu, hipStream_t s) {
 #define GEN(I, O, name) return launch_generic<I, O>(p, cu, s, name)
   if (in_dtype == IRIS_HIP_BF16 && out_dtype == IRIS_HIP_BF16) GEN(ElemBF16, ElemBF16, "generic_bf16");
@@ -390,6 +401,7 @@ void heap_bases_from_registry(FusedParams& p, const int64_t* context_tensor) {
 
 #ifdef IRIS_HIP_PHASE_STAMPS
 unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels record their phase stamps
+long long g_stamp_rows = 0;              // ... and how many rows of 16 words the buffer holds
 #endif
 
 // Launches for the 32x32 kernel (decode_kernel.h): any output small enough that it has at most two 32x32
@@ -401,8 +413,12 @@ unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels 
 // Beyond two tiles per CU the 64x64 tiled kernel is ahead at every K (fp16, 192x2880x4096: 25.0 against 29.4 us
 // for this kernel in a round of two and a round of one per CU; 640x1024x4096: 26.7 against 35.1; 32x32768x4096:
 // 51 against 66).
-bool decode_sized(const FusedParams& p, int cu_count) {
-  return (long long)cdiv(p.M, 32) * cdiv(p.N, 32) <= 2ll * cu_count;
+bool decode_sized(const FusedParams& p, int cu_count, int in_dtype) {
+  if ((long long)cdiv(p.M, 32) * cdiv(p.N, 32) > 2ll * cu_count) return false;
+  // ... and whose operands that kernel's 32-bit offsets reach (a tall A with long or padded rows does not
+  // qualify: 16384 x 32 outputs of K = 65536 bf16 have 2 GiB of A).
+  const long long a_rows = p.gather == GATHER_M ? p.M_local : p.M;
+  return decode_offsets_fit(a_rows, p.s_am, p.K_local, in_dtype == IRIS_HIP_FP8_E4M3 ? 1 : 2, p.M + p.row_offset, p.s_cm, p.N);
 }
 // ... and whose A that kernel can fetch: not gathered, gathered by rows in whole 32-row tiles per slot, or
 // gathered along K with every wave's 256 bytes of K inside one slot.
@@ -413,10 +429,12 @@ bool decode_gather_ok(const FusedParams& p, int in_dtype) {
   return true;
 }
 
-int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream) {
+// check_only: run every argument check and the kernel choice, launch nothing (0 = the launch would go out).
+int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream, bool check_only = false) {
   g_last_error[0] = 0;
 #ifdef IRIS_HIP_PHASE_STAMPS
   p.stamps = g_stamps;
+  p.stamp_rows = g_stamp_rows;
 #endif
   if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("M, N, K must be positive (got %d, %d, %d)", p.M, p.N, p.K);
   if (!p.A || !p.B || !p.C) return fail("A, B and C must not be NULL");
@@ -452,7 +470,7 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
   const bool rows64_ok = !(p.gather == GATHER_M && p.M_local % 64);
   int kind = TILE_SMALL;
   if (big_tiles * 100 >= (long long)facts->cu_count * 53 && !(p.M <= 64 && rows64_ok)) kind = TILE_BIG;
-  else if (decode_sized(p, facts->cu_count) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
+  else if (decode_sized(p, facts->cu_count, in_dtype) && decode_gather_ok(p, in_dtype) && p.world <= 8) kind = TILE_DECODE;
   else if ((long long)cdiv(p.M, 64) * cdiv(p.N, 64) <= 2ll * facts->cu_count && rows64_ok) kind = TILE_SKINNY64;
   else if (rows64_ok && (p.M <= 64 || ((long long)cdiv(p.M, 64) * cdiv(p.N, 128) <= 2ll * facts->cu_count &&
                                        (long long)p.K * elem_size(in_dtype) <= 2048)))
@@ -475,7 +493,11 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
     kind = forced_tile;  // a tile the operands do not qualify for is not forced
   const char* why = mfma_ineligible(p, in_dtype, out_dtype, tile_rows(kind), tile_cols(kind));
   if (path == IRIS_HIP_PATH_MFMA && why) return fail("MFMA kernel not applicable: %s", why);
-  if (path == IRIS_HIP_PATH_GENERIC || why) return dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
+  if (path == IRIS_HIP_PATH_GENERIC || why) {
+    if (!generic_supported(in_dtype, out_dtype)) return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
+    return check_only ? 0 : dispatch_generic(p, in_dtype, out_dtype, facts->cu_count, s);
+  }
+  if (check_only) return 0;
 
   const bool bkc = (p.s_bn != 1);
   switch (in_dtype) {
@@ -488,6 +510,35 @@ int run_fused(FusedParams p, int in_dtype, int out_dtype, int path, void* stream
 }
 
 bool fits_int(int64_t v) { return v > 0 && v < (1ll << 31); }
+
+// iris_hip_matmul_all_reduce; check_only stops in front of the launch (see run_fused).
+int matmul_all_reduce_impl(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
+                               int64_t M, int64_t N, int64_t K,
+                               int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                               int64_t stride_cm, int64_t stride_cn,
+                               const int64_t* context_tensor, int32_t cur_rank, int32_t world_size,
+                               int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
+                               int32_t variant, int32_t in_dtype, int32_t out_dtype, float scale,
+                               int32_t acc_mode, int64_t spin_limit, int32_t* status, int32_t path,
+                               void* stream, bool check_only) {
+  (void)block_size_k;
+  if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
+  if (variant != IRIS_HIP_VARIANT_ATOMIC && variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
+    return fail("variant %d is not atomic (0), one_shot (2) or two_shot (3)", variant);
+  FusedParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C; p.aux = (char*)aux_buffer; p.locks = locks;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.K_local = (int)K; p.gather = GATHER_NONE;
+  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
+  p.s_cm = stride_cm; p.s_cn = stride_cn;
+  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
+  p.rank = cur_rank; p.world = world_size;
+  p.flag_bm = block_size_m; p.flag_bn = block_size_n;
+  p.epi = variant == IRIS_HIP_VARIANT_ATOMIC ? EPI_ATOMIC : variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
+  p.acc_mode = acc_mode; p.all_owners = 0; p.sum_peers = 1;
+  p.scale = scale; p.spin_limit = spin_limit; p.status = status;
+  return run_fused(p, in_dtype, out_dtype, path, stream, check_only);
+}
 
 }  // namespace
 
@@ -527,23 +578,9 @@ int iris_hip_matmul_all_reduce(const void* A, const void* B, void* C, void* aux_
                                int32_t variant, int32_t in_dtype, int32_t out_dtype, float scale,
                                int32_t acc_mode, int64_t spin_limit, int32_t* status, int32_t path,
                                void* stream) {
-  (void)block_size_k;
-  if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
-  if (variant != IRIS_HIP_VARIANT_ATOMIC && variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
-    return fail("variant %d is not atomic (0), one_shot (2) or two_shot (3)", variant);
-  FusedParams p;
-  memset(&p, 0, sizeof(p));
-  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C; p.aux = (char*)aux_buffer; p.locks = locks;
-  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.K_local = (int)K; p.gather = GATHER_NONE;
-  p.s_am = stride_am; p.s_ak = stride_ak; p.s_bk = stride_bk; p.s_bn = stride_bn;
-  p.s_cm = stride_cm; p.s_cn = stride_cn;
-  p.heap_bases = context_tensor ? (const long long*)(context_tensor + 2) : nullptr;
-  p.rank = cur_rank; p.world = world_size;
-  p.flag_bm = block_size_m; p.flag_bn = block_size_n;
-  p.epi = variant == IRIS_HIP_VARIANT_ATOMIC ? EPI_ATOMIC : variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
-  p.acc_mode = acc_mode; p.all_owners = 0; p.sum_peers = 1;
-  p.scale = scale; p.spin_limit = spin_limit; p.status = status;
-  return run_fused(p, in_dtype, out_dtype, path, stream);
+  return matmul_all_reduce_impl(A, B, C, aux_buffer, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm,
+                                stride_cn, context_tensor, cur_rank, world_size, block_size_m, block_size_n, block_size_k,
+                                variant, in_dtype, out_dtype, scale, acc_mode, spin_limit, status, path, stream, false);
 }
 
 int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
@@ -560,6 +597,7 @@ int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, in
   const int es = elem_size(out_dtype);
   if (es == 0) return fail("unsupported element types in=%d out=%d", in_dtype, out_dtype);
   if (stride_cm < 0 || stride_cn < 0) return fail("negative output strides are not supported");
+  if (stride_cm >= (1ll << 40) || stride_cn >= (1ll << 40)) return fail("output strides beyond 2^40 elements are not supported");
   // aux is addressed with C's strides: the bytes it spans and the flags of the tile grid must fit.
   const long long aux_bytes = ((long long)(M - 1) * stride_cm + (long long)(N - 1) * stride_cn + 1) * es;
   const long long nflags = (long long)cdiv((int)M, block_size_m) * cdiv((int)N, block_size_n);
@@ -577,6 +615,12 @@ int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, in
   long long* context = (long long*)base;
   int32_t* locks = (int32_t*)(base + kScratchContextBytes);
   void* aux = base + kScratchAuxOffset;
+  // Every check of the launch itself (types, path, strides) before the prepare kernel goes out: a rejected
+  // call enqueues nothing and leaves the workspace alone.
+  rc = matmul_all_reduce_impl(A, B, C, aux, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm, stride_cn,
+                              (const int64_t*)context, 0, 1, block_size_m, block_size_n, block_size_k, variant, in_dtype,
+                              out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream, true);
+  if (rc) return rc;
   const int threads = 256;
   const int need = (int)nflags > (int)(kScratchContextBytes / sizeof(long long)) ? (int)nflags : (int)(kScratchContextBytes / sizeof(long long));
   hipLaunchKernelGGL(noalloc_prepare_kernel, dim3((need + threads - 1) / threads), dim3(threads), 0, (hipStream_t)stream,
@@ -729,8 +773,13 @@ int iris_hip_query(int32_t device, int32_t* cu_count, int32_t* xcc_count, int32_
 }
 
 #ifdef IRIS_HIP_PHASE_STAMPS
-// Diagnostic build only: device buffer of 16 x (number of workgroups) 64-bit words, or NULL.
-void iris_hip_debug_set_stamps(void* device_buffer) { g_stamps = (unsigned long long*)device_buffer; }
+// Diagnostic build only: device buffer of `rows` rows of 16 64-bit words, or NULL.  A launch writes row
+// it * (number of workgroups) + (workgroup) for the first eight tiles `it` of every workgroup; rows beyond
+// the buffer are not written.
+void iris_hip_debug_set_stamps(void* device_buffer, long long rows) {
+  g_stamps = (unsigned long long*)device_buffer;
+  g_stamp_rows = device_buffer ? rows : 0;
+}
 #endif
 
 const char* iris_hip_last_error(void) { return g_last_error; }

@@ -182,4 +182,17 @@ IRIS_HD int macro_tiles_over_flag_tile(int fm, int fn, int FM, int FN, int KM, i
   return nm * nn;
 }
 
+// The 32x32 small-output kernel addresses A from the operand's first row (of the slot that holds it) and
+// the peers' aux tiles from the buffer's first element, with 32-bit byte offsets into a buffer resource
+// of 2^31 bytes: an offset at or beyond 2^31 would read zeros.  True when every offset the kernel can
+// form stays below that: a_rows rows of A (the rows one slot holds) with a stride of s_am elements of es
+// bytes and K elements per row; M x N outputs of 2-byte elements with a row stride of s_cm elements.
+// Launches that fail the test take the tiled kernels, which rebase their resources per tile.
+IRIS_HD bool decode_offsets_fit(long long a_rows, long long s_am, long long K, int es, long long M, long long s_cm, long long N) {
+  const long long limit = 1ll << 31;
+  const long long a_last = (a_rows - 1) * s_am * es + K * es;  // one past the last byte of A
+  const long long c_last = ((M - 1) * s_cm + N) * 2;            // ... of aux / C
+  return a_rows > 0 && s_am >= 0 && s_cm >= 0 && a_last < limit && c_last < limit;
+}
+
 }  // namespace iris_layout

@@ -11,6 +11,7 @@ initialised, else to a world of one.  All W heaps are slots of one GPU allocatio
 import ctypes
 import logging
 import os
+import weakref
 
 import torch
 import torch.distributed as _dist
@@ -22,6 +23,16 @@ from .logging import logger
 # int64 words the reference appends for device-side tracing (iris/host/iris.py:916-958); kept as
 # zeros so the context tensor has the reference's length.
 _TRACE_WORDS = 17
+
+
+def _unregister_context(ptr):
+    """Drop the kernel library's record of the context tensor that lived at address `ptr`."""
+    try:
+        from .. import _lib
+
+        _lib.library().iris_hip_unregister_context(ctypes.c_void_p(ptr))
+    except Exception:  # interpreter shutdown: the library may be gone already
+        pass
 
 
 def _world_from_environment(num_ranks, rank):
@@ -239,6 +250,7 @@ class Iris:
         return self.heap_bases
 
     def _build_device_context(self):
+        self._forget_device_context()  # a context rebuilt in place drops its old entry first
         data = [self.cur_rank, self.num_ranks] + self.heap_bases.tolist() + [0] * _TRACE_WORDS
         host = torch.tensor(data, dtype=torch.int64)
         self._device_context = host.to(self.heap.device)
@@ -248,16 +260,21 @@ class Iris:
             # context tensor holds (one dependent load less on the way to the peers' flags).
             from .. import _lib
 
-            err = _lib.library().iris_hip_register_context(ctypes.c_void_p(self._device_context.data_ptr()),
-                                                           ctypes.c_void_p(host.data_ptr()), host.numel())
-            self._context_registered = err == 0
+            ptr = self._device_context.data_ptr()
+            err = _lib.library().iris_hip_register_context(ctypes.c_void_p(ptr), ctypes.c_void_p(host.data_ptr()),
+                                                           host.numel())
+            if err == 0:
+                # The registry is keyed by the tensor's address, and torch hands freed addresses out
+                # again: the entry goes away with the tensor (also at interpreter exit, also when
+                # __del__ never runs), so that no later tensor at this address inherits these bases.
+                self._context_finalizer = weakref.finalize(self._device_context, _unregister_context, ptr)
+                self._context_registered = True
 
     def _forget_device_context(self):
-        if getattr(self, "_context_registered", False):
-            from .. import _lib
-
-            _lib.library().iris_hip_unregister_context(ctypes.c_void_p(self._device_context.data_ptr()))
-            self._context_registered = False
+        finalizer = getattr(self, "_context_finalizer", None)
+        if finalizer is not None:
+            finalizer()  # idempotent: unregisters once
+        self._context_registered = False
 
     def get_device_context(self):
         """int64 tensor [cur_rank, W, heap_base_0..heap_base_{W-1}, 0 x 17] on the Iris device."""

@@ -228,6 +228,20 @@ void check_flag_counts() {
     }
 }
 
+// The rule that keeps launches away from the 32x32 kernel when its 32-bit offsets would not reach.
+void check_decode_offsets() {
+  CHECK(decode_offsets_fit(32, 1024, 1024, 1, 32, 8192, 8192), "decode shape 32 x 8192 x 1024 fp8");
+  CHECK(decode_offsets_fit(16384, 4096, 4096, 2, 16384, 32, 32), "tall output, 128 MiB of A");
+  CHECK(!decode_offsets_fit(16384, 65536, 65536, 2, 16384, 32, 32), "16384 x 65536 bf16 is 2 GiB of A");
+  CHECK(decode_offsets_fit(16384, 65536, 65536, 1, 16384, 32, 32), "the same in fp8 is 1 GiB");
+  CHECK(!decode_offsets_fit(2048, 1 << 20, 512, 2, 2048, 32, 32), "padded A rows: 2048 rows of 2 MiB");
+  CHECK(decode_offsets_fit(1023, 1 << 20, 512, 2, 1023, 32, 32), "1023 rows of 2 MiB end below 2 GiB");
+  CHECK(!decode_offsets_fit(1025, 1 << 20, 512, 2, 1025, 32, 32), "1025 rows of 2 MiB do not");
+  CHECK(!decode_offsets_fit(64, 512, 512, 2, 16385, 1 << 16, 32), "strided C view: 16385 rows of 128 KiB");
+  CHECK(decode_offsets_fit(64, 512, 512, 2, 16384, 1 << 15, 32), "16384 rows of 64 KiB end below 2 GiB");
+  CHECK(!decode_offsets_fit(0, 512, 512, 2, 64, 64, 64), "no rows");
+}
+
 int main() {
   check_row_tile<64>(256);
   check_row_tile<128>(256);
@@ -246,6 +260,7 @@ int main() {
   check_acc_layout();
   check_tile_orders();
   check_flag_counts();
+  check_decode_offsets();
   if (failures) { printf("%d check(s) failed\n", failures); return 1; }
   printf("layout_sim: all checks passed\n");
   return 0;

@@ -496,17 +496,18 @@ def test_peer_flags_raised_while_the_kernel_waits(M, N, K, variant):
             ctx.peer_view(ws.aux_buffer, r).copy_(peers[r])
             ctx.peer_view(ws.locks, r).zero_()
     torch.cuda.synchronize()
-    # Streams share a few hardware queues, and work behind the polling kernel in its own queue would only
-    # run once the kernel has given up: the flags are raised from four streams, which covers every queue
-    # (raising them twice is harmless).
-    sides = [torch.cuda.Stream() for _ in range(4)]
+    # The side stream's work goes out BEFORE the fused launch: a spin kernel, then the stores that raise the
+    # flags.  Whatever hardware queue the side stream shares, the spin kernel is already dispatched when
+    # the fused launch arrives, so nothing can queue the flag stores behind the polling kernel: either
+    # the two streams run side by side (the fused kernel polls until the spin kernel ends) or the fused
+    # launch waits behind both (and finds the flags up).
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(2_000_000)
+        for r in range(W):
+            if r != rank:
+                ctx.peer_view(ws.locks, r).fill_(1)
     ops.matmul_all_reduce(ctx, dC, dA, dB, async_op=True, config=cfg, workspace=ws)
-    for side in sides:
-        with torch.cuda.stream(side):
-            torch.cuda._sleep(2_000_000)  # the launch above is polling by now
-            for r in range(W):
-                if r != rank:
-                    ctx.peer_view(ws.locks, r).fill_(1)
     torch.cuda.synchronize()
     ctx.check_status()  # no spin time-out
     exp = oracle.matmul_all_reduce(A, B, peers, rank, W, fbm, 64, variant, "fp32")

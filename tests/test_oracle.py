@@ -424,3 +424,20 @@ def test_ccl_two_shot_matches_the_program_loop(comm_sms, distribution):
         differs += int(np.sum(ascending[own] != want[own]))
     assert np.all(covered == 1)
     assert differs > 50, "the data must tell the rotated order from the ascending one"
+
+
+def test_rel_frobenius_known_answers():
+    """The yardstick of every tolerance test: ||x - ref||_F / ||ref||_F, worked by hand.
+    ref = [[3, 4]] has norm 5; x = ref + [[0.3, -0.4]] is off by a vector of norm 0.5: 0.1.  The measure
+    is relative to the SECOND argument (swapping the arguments gives 0.5 / ||x||, another number), is 0
+    for equal inputs, sees every element (a single wrong entry of a 2x2 identity: 1 / sqrt(2)), works
+    across dtypes in float64, and falls back to the absolute error for a zero reference."""
+    ref = torch.tensor([[3.0, 4.0]])
+    x = torch.tensor([[3.3, 3.6]])
+    assert oracle.rel_frobenius(x, ref) == pytest.approx(0.1, rel=1e-6)
+    assert oracle.rel_frobenius(ref, x) == pytest.approx(0.5 / (3.3 ** 2 + 3.6 ** 2) ** 0.5, rel=1e-6)
+    assert oracle.rel_frobenius(ref, ref) == 0.0
+    eye, bad = torch.eye(2), torch.tensor([[1.0, 0.0], [1.0, 1.0]])
+    assert oracle.rel_frobenius(bad, eye) == pytest.approx(2 ** -0.5, rel=1e-12)
+    assert oracle.rel_frobenius(torch.tensor([2.5], dtype=torch.bfloat16), torch.tensor([2.0])) == pytest.approx(0.25)
+    assert oracle.rel_frobenius(torch.tensor([0.0, 2.0]), torch.zeros(2)) == pytest.approx(2.0)
