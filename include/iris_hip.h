@@ -22,7 +22,8 @@
  *   - Launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
  *   - Return value: 0 on success, otherwise a hipError_t value.  Argument errors return
  *     hipErrorInvalidValue (1); iris_hip_last_error() then describes the problem.
- *   - The library calls no hipMalloc.  It keeps between calls: device facts (CU count, XCD count, LDS
+ *   - The library calls hipMalloc only for the split-tile workspace described at iris_hip_set_split_tiles
+ *     (iris_hip_matmul_all_reduce_noalloc never does).  It keeps between calls: device facts (CU count, XCD count, LDS
  *     size) cached per device under a mutex, a once-per-device "attribute set" flag per kernel build
  *     (atomic), the last error and last kernel name per host thread, the contents of context tensors
  *     registered with iris_hip_register_context (under a mutex), and one static device array that
@@ -282,6 +283,22 @@ int iris_hip_reduce_scatter(const void* input, void* output, int64_t M, int64_t 
  */
 int iris_hip_register_context(const int64_t* context_tensor, const int64_t* host_copy, int32_t num_words);
 int iris_hip_unregister_context(const int64_t* context_tensor);
+
+/*
+ * Tail policy of the 256x256 tile (no counterpart in the reference, whose persistent schedule hands
+ * tiles out whole: iris/ops/all_gather_matmul.py:71-79).  When the tile count leaves the last round of
+ * workgroups partly empty for many K steps, the K steps of that round's tiles are shared out evenly
+ * between all workgroups; a tile that ends up in several shares is summed from fp32 partial sums that
+ * travel through a workspace of the library (64 MiB + 1 KiB per (device, stream), allocated with
+ * hipMalloc on the stream's first such launch, never under stream capture - a capturing stream without
+ * a workspace launches without splitting -, kept until the process ends, at most 8 per device).
+ * mode: -1 the library decides per launch (default: when the split round is expected to be at least 24 K
+ * steps and an eighth shorter than a whole tile), 0 never split, 1 split whenever the last round is not
+ * full and its tiles have at least 4 K steps (a test setting), 2 split whenever any gain is expected (a
+ * tuning aid).  The environment variable IRIS_HIP_STREAMK sets the initial mode.  A split launch differs
+ * from an unsplit one only in the order of the fp32 sums over K.
+ */
+void iris_hip_set_split_tiles(int32_t mode);
 
 /*
  * Device facts used by the host layer (reference: get_cu_count / get_num_xcc,

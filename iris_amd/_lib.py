@@ -85,6 +85,7 @@ PROTOTYPES = {
     "iris_hip_register_context": (_i32, [_ptr, _ptr, _i32]),
     "iris_hip_unregister_context": (_i32, [_ptr]),
     "iris_hip_query": (_i32, [_i32, _ptr, _ptr, _ptr]),
+    "iris_hip_set_split_tiles": (None, [_i32]),
     "iris_hip_last_error": (ctypes.c_char_p, []),
     "iris_hip_last_kernel": (ctypes.c_char_p, []),
     "iris_hip_abi_version": (_i32, []),

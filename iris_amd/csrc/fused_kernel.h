@@ -68,6 +68,13 @@ struct FusedParams {
   // on the way to the peers' flags and tiles.
   long long hb_arg[8];
   int hb_in_args;
+  // Split tiles (see the STREAMK builds of fused_mfma_kernel): one slot of partial sums and one flag per
+  // workgroup, and the value a flag takes in this launch.  NULL / 0 when the launch does not split tiles.
+  char* sk_partials;
+  int* sk_flags;
+  int sk_epoch;
+  int sk_gather_cost, sk_pass_cost;  // the costs the host planned the split with (iris_layout::split_plan)
+  int no_workspace_alloc;  // host only: the caller must not trigger an allocation (split tiles need one)
 #ifdef IRIS_HIP_PHASE_STAMPS
   unsigned long long* stamps;  // diagnostic build: rows of 16 time stamps (see PHASE_STAMP)
   long long stamp_rows;        // rows the buffer holds; rows beyond it are not written
@@ -229,7 +236,9 @@ struct MfmaCfg {
   // the accumulator-layout writes (one row per lane) spread over the LDS banks.
   static constexpr int TROW = BN * 2 + 16;
   static constexpr int TILE_BYTES = BM * TROW;
-  static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES;
+  // One word per wave behind the staged tile, for workgroup-wide votes in the epilogue (workgroup_all).
+  static constexpr int VOTE_OFFSET = TILE_BYTES;
+  static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES + 64 ? RING_BYTES : TILE_BYTES + 64;
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
   // Four-wave tiles whose ring fits twice into a CU's LDS run two workgroups per CU, so that the
   // memory round trips of one workgroup's epilogue hide behind the other's K loop.
@@ -290,6 +299,15 @@ __device__ __forceinline__ void store16_system(char* p, u32x4_t v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
 }
 
+// The same for data that the next instructions overwrite with VALU results (accumulator reads, say):
+// a store of more than 8 bytes is still fetching its data registers for the last lanes when the next
+// instruction issues, and a VALU write to them in that slot reaches memory for those lanes.  The
+// compiler pads this hazard between instructions it can see; it cannot see into the asm statement, so
+// the wait states are part of it.
+__device__ __forceinline__ void store16_system_of_valu_data(char* p, u32x4_t v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+}
+
 // Read one accumulator register.  The "a" constraint keeps the MFMA results in the accumulation
 // registers until the epilogue consumes them, instead of copying all of them to VGPRs at once.
 __device__ __forceinline__ float acc_read(float a) {
@@ -298,8 +316,32 @@ __device__ __forceinline__ float acc_read(float a) {
   return v;
 }
 
+// a += x for a value that lives in an accumulation register, without the compiler moving the tile's
+// accumulators to VGPRs to do it.
+__device__ __forceinline__ float acc_add(float a, float x) {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_add_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1" : "+a"(a), "=&v"(t) : "v"(x));
+  return a;
+}
+
 __device__ __forceinline__ unsigned lds_address(const void* p) {
   return (unsigned)(unsigned long long)(LDS_AS const char*)p;
+}
+
+// True when `pred` holds in every thread of the workgroup; doubles as a workgroup barrier (two of them).
+// The votes of the waves meet in `words` (one int per wave, LDS that nothing else uses at this point).
+// Unlike __syncthreads_and it takes no static LDS of its own, which would come on top of the dynamic
+// LDS and so cap the operand ring one KiB short of the CU's 160 KiB.
+template <int NW>
+__device__ __forceinline__ bool workgroup_all(bool pred, char* words, int wave, int lane) {
+  const int mine = __all(pred) ? 1 : 0;
+  if (lane == 0) *(LDS_AS int*)(LDS_AS char*)(words + 4 * wave) = mine;
+  __syncthreads();
+  int all = 1;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) all &= *(const LDS_AS int*)(LDS_AS char*)(words + 4 * w);
+  __syncthreads();  // the words may be rewritten (next tile's vote) only after everybody has read them
+  return all != 0;
 }
 
 template <class CFG>
@@ -381,8 +423,19 @@ __device__ __forceinline__ FusedParams pin_loader_arguments(const FusedParams& a
 // ONE_ROUND: the launch has a workgroup for every tile, so a workgroup handles at most one.  The
 // tile loop is then known to run once, which lets the compiler drop everything it otherwise carries
 // from tile to tile (measured: 1.2 us of a 9 us launch on decode-sized problems).
-template <class CFG, bool ONE_ROUND>
+//
+// STREAMK (eight-wave tile only): the tail policy for tile counts that do not fill the last round of
+// workgroups (iris_layout::split_plan has the scheme).  Inside every XCD's span of tiles, the tiles of
+// the full rounds are handed out whole, as in the other builds.  In the last round the workgroups that
+// would find no tile help the others: a helper multiplies a piece of a tile's K steps, stores its fp32
+// accumulators to the piece's slot of p.sk_partials (write-through) and sets the slot's flag to
+// p.sk_epoch; the tile's main workgroup multiplies the first K steps, waits for its helpers' flags, adds
+// their partial sums in ascending piece order and runs the ordinary epilogue.  Helpers are the XCD's
+// first workgroups and never wait, mains wait only for helpers - workgroups with lower indices, which
+// the hardware dispatches first - so the waits end whatever part of the grid is resident.
+template <class CFG, bool ONE_ROUND, bool STREAMK = false>
 __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kernel(const FusedParams p_in) {
+  static_assert(!STREAMK || (CFG::NW == 8 && !ONE_ROUND), "split tiles: eight-wave tile, looping build");
   using Out = typename OutOf<CFG::IN>::type;
   using ATile = RowTile<CFG::RBA>;
   constexpr int ES = CFG::ES, CE = CFG::CE, BM = CFG::BM, BN = CFG::BN, BK = CFG::BK;
@@ -547,9 +600,44 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   const unsigned smem_base = __builtin_amdgcn_readfirstlane(lds_address(smem));
   const unsigned long long a_own = (unsigned long long)p.A;
 
+  // Split tiles (iris_layout::split_plan): every workgroup first takes its whole tiles, dp_rounds of
+  // them at positions dp_first + round * wg_per_xcd of the grouped order; then the last round's tiles,
+  // at positions sk_first + j, go to a main and its helpers.  Partial sum slot (and flag) of piece i >= 1
+  // of tile j: sk_slot0 + j * per_tile + i - 1.
+  enum { ITEM_WHOLE = 0, ITEM_PART = 1, ITEM_OWNER = 2 };  // the kinds of iris_layout::split_item
+  int sk_first = 0, sk_left = 0, sk_slot0 = 0, sk_served = 0, dp_first = 0, dp_rounds = 0, dp_it = 0, wg_per_xcd = 1, sk_local = 0;
+  SplitPlan plan = {0, 1, nsteps, 0};
+  if constexpr (STREAMK) {
+    const int xcd = blockIdx.x % p.num_xcd;
+    sk_local = blockIdx.x / p.num_xcd;
+    wg_per_xcd = gridDim.x / p.num_xcd;
+    const int span = cdiv(total_tiles, p.num_xcd);
+    const int first = min(xcd * span, total_tiles);
+    const int mine = min(span, total_tiles - first);  // tiles of this XCD
+    dp_rounds = mine / wg_per_xcd;
+    sk_left = mine - dp_rounds * wg_per_xcd;          // tiles of the last, partly filled round
+    dp_first = first + sk_local;
+    sk_first = first + dp_rounds * wg_per_xcd;
+    sk_slot0 = xcd * wg_per_xcd;
+    plan = split_plan(sk_left, wg_per_xcd, nsteps, p.sk_gather_cost, p.sk_pass_cost);
+  }
+
   for (int it = 0; ONE_ROUND ? it < 1 : true; ++it) {
-    const int tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
-    if (tidx < 0) break;
+    int tidx, k_begin = 0, k_end = nsteps, item = ITEM_WHOLE, partners = 0, slot = 0;
+    if constexpr (STREAMK) {
+      if (dp_it < dp_rounds) {
+        tidx = dp_first + dp_it * wg_per_xcd;
+        ++dp_it;
+      } else {
+        int j;
+        if (!split_item(plan, sk_left, wg_per_xcd, nsteps, sk_local, sk_served++, j, k_begin, k_end, item, partners, slot)) break;
+        tidx = sk_first + j;
+        slot += sk_slot0;
+      }
+    } else {
+      tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
+      if (tidx < 0) break;
+    }
     PHASE_STAMP(0);
     int tm, tn;
     grouped_tile(tidx, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
@@ -574,13 +662,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       a_slot = m0 / p.M_local;
       a_row0 = m0 - (long long)a_slot * p.M_local;
     }
-    if (p.gather == GATHER_K) a_slot = 0;
+    if (p.gather == GATHER_K) a_slot = k_begin / nkb;  // the source that holds the first K step
     const unsigned long long a_tile_off = (unsigned long long)(a_row0 * p.s_am * ES);
     const i32x4_t rb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)n0 * (CFG::B_KCONTIG ? p.s_bn : 1) * ES);
     i32x4_t ra = make_rsrc_words((p.gather == GATHER_NONE ? a_own : in_slot(a_own, a_slot)) + a_tile_off);
 
     // Loader position: next K step to issue = (i_src, i_kb), i_step overall.
-    int i_step = 0, i_src = 0, i_kb = 0;
+    int i_step = k_begin, i_src = k_begin / nkb, i_kb = k_begin - (k_begin / nkb) * nkb;
 
     // The direct-to-LDS loads of one K step, issued one at a time so that the main loop can spread
     // them between its MFMAs (a wave issues in order: a burst of loads right after the barrier would
@@ -593,7 +681,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     };
     auto begin_step = [&](int slot_off) {  // slot_off: byte offset of the ring slot to fill
       StepLoads L;
-      const bool live = i_step < nsteps;
+      const bool live = i_step < k_end;
       const int k0 = i_kb * BK;
       L.klim = live ? klocal - k0 : 0;  // k elements of this step that exist
       L.sa = smem_base + slot_off + wave * kDmaBytes;
@@ -660,7 +748,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     // which turns every LDS address of a step into a constant offset (5-10 % on those tiles); the
     // eight-wave tile would spill and keeps the ring position in a register.
     constexpr int RING_UNROLL = (NW == 4) ? STAGES : 1;
-    int s = 0, ring_pos = 0;
+    int s = k_begin, ring_pos = 0;
     if constexpr (PINGPONG) {
       // Eight waves, two per SIMD: waves 0-3 and waves 4-7 run half a step apart.  A step is a
       // memory phase (all fragment reads of the step, then the direct-to-LDS loads that refill the
@@ -681,7 +769,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         const long long kglob = (long long)i_src * klocal + (long long)i_kb * BK;
         b_so = __builtin_amdgcn_readfirstlane(
             CFG::B_KCONTIG ? (unsigned)(kglob * ES) : (unsigned)(kglob * p.s_bk * ES));
-        k_left = i_step < nsteps ? klocal - i_kb * BK : 0;
+        k_left = i_step < k_end ? klocal - i_kb * BK : 0;
       };
       resync();
       unsigned rd = 0;                                    // byte offset of the slot this step reads
@@ -708,7 +796,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           load_frags_a(fr[0], rd, 0, MB / 2 + pc);
         }
       };
-      for (; s < nsteps; ++s) {
+      for (; s < k_end; ++s) {
         if constexpr (SPLIT_K) {
 #pragma unroll
           for (int kk = 0; kk < KS / 2; ++kk) load_frags(fr[kk], rd, kk);
@@ -765,10 +853,10 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       }
       if (!late) __builtin_amdgcn_s_barrier();
     } else
-    while (s < nsteps) {
+    while (s < k_end) {
 #pragma unroll
     for (int u = 0; u < RING_UNROLL; ++u) {
-      if (s >= nsteps) break;
+      if (s >= k_end) break;
       ++s;
       const int slot = (RING_UNROLL == 1) ? ring_pos : u;
       // LDS is one coherent memory per CU, so a bare s_barrier (no fence, hence no forced wait for
@@ -816,11 +904,56 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     __syncthreads();
     PHASE_STAMP(2);
 
+    if constexpr (STREAMK) {
+      // Partial sums travel in the accumulators' own layout: 16-byte piece j of thread t at byte
+      // (j * NT + t) * 16 of the workgroup's slot, so that every wave instruction moves 1 KiB.
+      constexpr int PIECES = MB * NB * 4;  // 16-byte pieces per thread
+      constexpr long long SLOT_BYTES = (long long)PIECES * NT * 16;
+      if (item == ITEM_PART) {
+        // (The base goes through an empty asm so that the compiler computes the pieces' addresses here, one
+        // at a time, instead of keeping all of them in registers from the top of the kernel.)
+        unsigned long long slot_base = (unsigned long long)p.sk_partials + (unsigned long long)slot * SLOT_BYTES;
+        asm volatile("" : "+s"(slot_base));
+        char* const dst = (char*)slot_base + tid * 16;
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) {
+          const int mb = j / (NB * 4), nb = (j / 4) % NB, q = j % 4;
+          u32x4_t v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = __float_as_uint(acc_read(acc.v[mb][nb][4 * q + e]));
+          store16_system_of_valu_data(dst + (long long)j * NT * 16, v);
+          __builtin_amdgcn_sched_barrier(0);  // one piece at a time: the scheduler would read all 128 registers first
+        }
+        // Published like an aux tile: stores acknowledged by every wave, then one relaxed flag store.
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (tid == 0) __hip_atomic_store(p.sk_flags + slot, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        continue;  // the ring is free (barrier above); no epilogue for a partial sum
+      }
+      if (item == ITEM_OWNER) {
+        if (tid < partners) {
+          const int* flag = p.sk_flags + (slot + tid);
+          long long polls = 0;
+          while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != p.sk_epoch) {
+            if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
+              if (p.status) __hip_atomic_store(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+          }
+        }
+        __syncthreads();
+      }
+    }
+
     // ---- epilogue -------------------------------------------------------------------------------
     // The whole output tile is first written to LDS in the output type (the operand ring is dead
     // by now), which frees the accumulators; both phases then stream rows of the tile, 16 bytes per
     // lane and BN*2 contiguous bytes per row, with many loads in flight per thread.
     {
+      // Split tiles: 16-byte pieces of a partial sum, in the layout its workgroup stored them in.
+      constexpr int PIECES = MB * NB * 4, NBATCH = 4, BATCH = PIECES / NBATCH;
+      constexpr long long SLOT_BYTES = (long long)PIECES * NT * 16;
       float badd[MB];
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
@@ -830,22 +963,87 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           if (gm < p.M) badd[mb] = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
         }
       }
+      // Piece j of the thread: 4 consecutive n of one m, from their fp32 sums to the staged tile.
+      auto stage_piece = [&](int j, const float (&sum)[4]) {
+        const int mb = j / (NB * 4), nb = (j / 4) % NB, q = j % 4;
+        float h[4];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
+        for (int e = 0; e < 4; ++e) h[e] = sum[e] * p.scale + badd[mb];
+        u32x2_t w;
+        w.x = Out::pack(h[0], h[1]);
+        w.y = Out::pack(h[2], h[3]);
+        const int trow = wm * TM + mb * 32 + acc_col(lane);
+        const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
+        *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
+      };
+      auto own_piece = [&](int j, float (&sum)[4]) {
+        const int mb = j / (NB * 4), nb = (j / 4) % NB, q = j % 4;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
+        for (int e = 0; e < 4; ++e) sum[e] = acc_read(acc.v[mb][nb][4 * q + e]);
+      };
+      bool staged = false;
+      if constexpr (STREAMK) {
+        if (item == ITEM_OWNER) {
+          // own sum + the partners' partial sums in ascending workgroup order, a quarter of the pieces
+          // at a time.  (The accumulators are only read: adding into them in place makes the compiler
+          // move the whole tile through VGPRs.)
+          staged = true;
+          auto slot_of = [&](int pr) -> const char* {
+            unsigned long long base = (unsigned long long)p.sk_partials + (unsigned long long)(slot + pr) * SLOT_BYTES;
+            asm volatile("" : "+s"(base));  // addresses are formed where they are used, not hoisted out of the tile loop
+            return (const char*)base + tid * 16;
+          };
+          auto load_batch = [&](u32x4_t (&dst)[BATCH], const char* src, int b) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float h[4];
+            for (int i = 0; i < BATCH; ++i)
+              dst[i] = __builtin_nontemporal_load((const u32x4_t*)(src + (long long)(b * BATCH + i) * NT * 16));
+          };
+          if (partners == 1) {  // the usual case: the next batch is on its way while this one is staged
+            const char* const src = slot_of(0);
+            u32x4_t buf[2][BATCH];
+            load_batch(buf[0], src, 0);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = acc_read(acc.v[mb][nb][4 * q + e]) * p.scale + badd[mb];
-            u32x2_t w;
-            w.x = Out::pack(h[0], h[1]);
-            w.y = Out::pack(h[2], h[3]);
-            const int trow = wm * TM + mb * 32 + acc_col(lane);
-            const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
-            *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
+            for (int b = 0; b < NBATCH; ++b) {
+              if (b + 1 < NBATCH) load_batch(buf[(b + 1) & 1], src, b + 1);
+#pragma unroll
+              for (int i = 0; i < BATCH; ++i) {
+                float sum[4];
+                own_piece(b * BATCH + i, sum);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sum[e] += __uint_as_float(buf[b & 1][i][e]);
+                stage_piece(b * BATCH + i, sum);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          } else {
+#pragma unroll
+            for (int b = 0; b < NBATCH; ++b) {  // unrolled: accumulators are registers, their indices constants
+              float sum[BATCH][4];
+#pragma unroll
+              for (int i = 0; i < BATCH; ++i) own_piece(b * BATCH + i, sum[i]);
+#pragma unroll 1
+              for (int pr = 0; pr < partners; ++pr) {
+                u32x4_t buf[BATCH];
+                load_batch(buf, slot_of(pr), b);
+#pragma unroll
+                for (int i = 0; i < BATCH; ++i)
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) sum[i][e] += __uint_as_float(buf[i][e]);
+              }
+#pragma unroll
+              for (int i = 0; i < BATCH; ++i) stage_piece(b * BATCH + i, sum[i]);
+            }
           }
+        }
+      }
+      if (!staged) {
+#pragma unroll
+        for (int j = 0; j < PIECES; ++j) {
+          float sum[4];
+          own_piece(j, sum);
+          stage_piece(j, sum);
+        }
+      }
     }
     __syncthreads();
     PHASE_STAMP(3);
@@ -931,7 +1129,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // and the polling after the own flags are raised is skipped.
       const bool up_already = solo ? true : probe_peer_flags<BM, BN, NT>(p, m0, n0, tid);
       wait_vmcnt<0>();
-      const bool all_up = __syncthreads_and(up_already);
+      const bool all_up = workgroup_all<NW>(up_already, smem + CFG::VOTE_OFFSET, wave, lane);
       PHASE_STAMP(5);
       raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
       if (!solo) {
@@ -1103,20 +1301,50 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 // ------------------------------------------------------------------------------------------------
 // Launch of the MFMA kernel
 // ------------------------------------------------------------------------------------------------
-template <class CFG, bool ONE_ROUND>
+template <class CFG, bool ONE_ROUND, bool STREAMK = false>
 int launch_mfma_grid(const FusedParams& p, int device, int grid, hipStream_t stream) {
   // The dynamic-LDS limit is a per-device attribute of the kernel: set it once on every device used
   // (atomic flags: two host threads may both set it, which is harmless, but neither skips it).
   static std::atomic<bool> attr_set[64];
   if (device < 0 || device >= 64) return iris_host::fail("device index %d out of range", device);
   if (!attr_set[device].load(std::memory_order_acquire)) {
-    hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG, ONE_ROUND>,
+    hipError_t e = hipFuncSetAttribute((const void*)fused_mfma_kernel<CFG, ONE_ROUND, STREAMK>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, CFG::SMEM_BYTES);
     if (e != hipSuccess) return (int)e;
     attr_set[device].store(true, std::memory_order_release);
   }
-  hipLaunchKernelGGL((fused_mfma_kernel<CFG, ONE_ROUND>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
+  hipLaunchKernelGGL((fused_mfma_kernel<CFG, ONE_ROUND, STREAMK>), dim3(grid), dim3(CFG::NT), CFG::SMEM_BYTES, stream, p);
   return (int)hipGetLastError();
+}
+
+// Tail policy of the eight-wave tile (the STREAMK builds of the kernel): worth it when the last round of
+// workgroups would leave a good part of the chip without a tile for many K steps.  Returns the grid to
+// launch (every CU, a multiple of the XCD count) or 0 when tiles are better handed out whole.
+//   iris_hip_set_split_tiles(0) / IRIS_HIP_STREAMK=0 never splits, 1 splits whenever the last round is
+//   not full and has at least 4 K steps, -1 (default) decides by the rule below.  Results differ from the unsplit launch only in
+//   the order of the fp32 sums over K.
+template <class CFG>
+int split_tile_grid(FusedParams& p, int total, int cu_count) {
+  if constexpr (CFG::NW != 8) return 0;
+  const int mode = iris_host::split_tile_mode();
+  if (mode == 0 || p.no_workspace_alloc || p.num_xcd < 1) return 0;
+  const int grid = cu_count - cu_count % p.num_xcd;
+  if (grid < p.num_xcd) return 0;
+  const int wg_per_xcd = grid / p.num_xcd;
+  const int span = cdiv(total, p.num_xcd);     // tiles of an XCD (the last one may have fewer)
+  const int left = span % wg_per_xcd;          // tiles of its last, partly filled round
+  if (left == 0) return 0;
+  const int nsrc = p.gather == GATHER_K ? p.world : 1;
+  const int nsteps = nsrc * cdiv(p.gather == GATHER_K ? p.K_local : p.K, CFG::BK);
+  // Mode 1 plans without the costs of passing partial sums on: whatever can be split is split.
+  p.sk_gather_cost = mode == 1 ? 0 : kSplitGatherCost;
+  p.sk_pass_cost = mode == 1 ? 0 : kSplitPassCost;
+  const SplitPlan plan = split_plan(left, wg_per_xcd, nsteps, p.sk_gather_cost, p.sk_pass_cost);
+  if (plan.per_tile == 0) return 0;
+  if (mode == 1 || mode == 2) return grid;  // 2: whatever the plan expects any gain from (a tuning aid)
+  // Worth it when the split round is at least 24 K steps (18 us) and an eighth shorter than a whole tile.
+  const int steps = split_round_steps(plan, nsteps);
+  return (nsteps - steps >= 24 && (nsteps - steps) * 8 >= nsteps) ? grid : 0;
 }
 
 template <class CFG>
@@ -1132,6 +1360,23 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   }
   if (grid < 1) grid = 1;
   iris_host::set_last_kernel(name);
+  const bool uneven_tiles = p.epi == EPI_TWO_SHOT || (p.epi == EPI_REDUCE_SCATTER && !p.all_owners);
+  const bool per_tile_launch = uneven_tiles && p.world > 1 && p.sum_peers && total > grid;
+  if constexpr (CFG::NW == 8) {
+    FusedParams q = p;
+    const int sk_grid = per_tile_launch ? 0 : split_tile_grid<CFG>(q, total, cu_count);
+    if (sk_grid > 0) {
+      constexpr long long slot_bytes = (long long)CFG::MB * CFG::NB * 4 * CFG::NT * 16;
+      // No workspace (the stream is being captured before its first split launch, or the device has
+      // used up its workspaces): hand the tiles out whole.
+      if (iris_host::split_tile_workspace(device, stream, sk_grid, slot_bytes, &q.sk_partials, &q.sk_flags, &q.sk_epoch) == 0) {
+        char sk_name[112];
+        snprintf(sk_name, sizeof(sk_name), "%s_splitk", name);
+        iris_host::set_last_kernel(sk_name);
+        return launch_mfma_grid<CFG, false, true>(q, device, sk_grid, stream);
+      }
+    }
+  }
   if (total <= grid) return launch_mfma_grid<CFG, true>(p, device, grid, stream);
   // More tiles than workgroups that fit at once: normally the resident workgroups loop over the tiles.
   // The two-shot all-reduce does better with one workgroup per tile, handed out by the hardware as CUs
@@ -1140,8 +1385,7 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   // without peers do not care.  The same goes for a reduce-scatter whose rank owns one block of
   // rows: the few tiles that carry the slot sum take half as long again as the others, and a fixed
   // tile-to-workgroup assignment gives some workgroups two of them.
-  const bool uneven_tiles = p.epi == EPI_TWO_SHOT || (p.epi == EPI_REDUCE_SCATTER && !p.all_owners);
-  if (uneven_tiles && p.world > 1 && p.sum_peers) {
+  if (per_tile_launch) {
     int per_tile = total;
     if (per_tile % p.num_xcd) per_tile += p.num_xcd - per_tile % p.num_xcd;
     return launch_mfma_grid<CFG, true>(p, device, per_tile, stream);

@@ -30,6 +30,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -520,7 +521,7 @@ int matmul_all_reduce_impl(const void* A, const void* B, void* C, void* aux_buff
                                int32_t block_size_m, int32_t block_size_n, int32_t block_size_k,
                                int32_t variant, int32_t in_dtype, int32_t out_dtype, float scale,
                                int32_t acc_mode, int64_t spin_limit, int32_t* status, int32_t path,
-                               void* stream, bool check_only) {
+                               void* stream, bool check_only, bool no_alloc = false) {
   (void)block_size_k;
   if (!fits_int(M) || !fits_int(N) || !fits_int(K)) return fail("M, N, K must be in [1, 2^31)");
   if (variant != IRIS_HIP_VARIANT_ATOMIC && variant != IRIS_HIP_VARIANT_ONE_SHOT && variant != IRIS_HIP_VARIANT_TWO_SHOT)
@@ -537,6 +538,7 @@ int matmul_all_reduce_impl(const void* A, const void* B, void* C, void* aux_buff
   p.epi = variant == IRIS_HIP_VARIANT_ATOMIC ? EPI_ATOMIC : variant == IRIS_HIP_VARIANT_ONE_SHOT ? EPI_ONE_SHOT : EPI_TWO_SHOT;
   p.acc_mode = acc_mode; p.all_owners = 0; p.sum_peers = 1;
   p.scale = scale; p.spin_limit = spin_limit; p.status = status;
+  p.no_workspace_alloc = no_alloc ? 1 : 0;
   return run_fused(p, in_dtype, out_dtype, path, stream, check_only);
 }
 
@@ -555,6 +557,66 @@ int fail(const char* fmt, ...) {
 void clear_last_error() { g_last_error[0] = 0; }
 
 void set_last_kernel(const char* name) { snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", name); }
+
+namespace {
+struct SplitTileWorkspace {
+  int device;
+  hipStream_t stream;
+  char* partials;
+  int* flags;
+  int nwg;
+  long long slot_bytes;
+  unsigned epoch;
+};
+constexpr int kMaxSplitWorkspacesPerDevice = 8;
+std::vector<SplitTileWorkspace> g_split_workspaces;
+std::mutex g_split_mutex;
+}  // namespace
+
+namespace {
+std::atomic<int> g_split_mode{[] { const char* e = getenv("IRIS_HIP_STREAMK"); return e ? atoi(e) : -1; }()};
+}
+int split_tile_mode() { return g_split_mode.load(std::memory_order_relaxed); }
+void set_split_tile_mode(int mode) { g_split_mode.store(mode < 0 ? -1 : (mode > 2 ? 2 : mode), std::memory_order_relaxed); }
+
+int split_tile_workspace(int device, hipStream_t stream, int nwg, long long slot_bytes, char** partials, int** flags, int* epoch) {
+  std::lock_guard<std::mutex> lock(g_split_mutex);
+  int on_device = 0;
+  for (SplitTileWorkspace& w : g_split_workspaces) {
+    if (w.device != device) continue;
+    ++on_device;
+    if (w.stream != stream || w.nwg < nwg || w.slot_bytes < slot_bytes) continue;
+    w.epoch = w.epoch % 0x7FFFFFFFu + 1;  // 1 .. 2^31 - 1: never the 0 the flags start with
+    *partials = w.partials;
+    *flags = w.flags;
+    *epoch = (int)w.epoch;
+    return 0;
+  }
+  if (on_device >= kMaxSplitWorkspacesPerDevice) return 1;
+  // First split launch on this stream.  Nothing may be allocated or cleared on a stream under capture.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return 1;
+  }
+  SplitTileWorkspace w{device, stream, nullptr, nullptr, nwg, slot_bytes, 1u};
+  if (hipMalloc((void**)&w.partials, (size_t)nwg * (size_t)slot_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return 1;
+  }
+  if (hipMalloc((void**)&w.flags, (size_t)nwg * sizeof(int)) != hipSuccess ||
+      hipMemsetAsync(w.flags, 0, (size_t)nwg * sizeof(int), stream) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(w.partials);
+    if (w.flags) (void)hipFree(w.flags);
+    return 1;
+  }
+  g_split_workspaces.push_back(w);
+  *partials = w.partials;
+  *flags = w.flags;
+  *epoch = 1;
+  return 0;
+}
 
 int device_facts(int device, int* cu_count, int* xcc_count) {
   DeviceFacts* f = nullptr;
@@ -619,7 +681,7 @@ int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, in
   // call enqueues nothing and leaves the workspace alone.
   rc = matmul_all_reduce_impl(A, B, C, aux, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm, stride_cn,
                               (const int64_t*)context, 0, 1, block_size_m, block_size_n, block_size_k, variant, in_dtype,
-                              out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream, true);
+                              out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream, true, true);
   if (rc) return rc;
   const int threads = 256;
   const int need = (int)nflags > (int)(kScratchContextBytes / sizeof(long long)) ? (int)nflags : (int)(kScratchContextBytes / sizeof(long long));
@@ -627,9 +689,9 @@ int iris_hip_matmul_all_reduce_noalloc(const void* A, const void* B, void* C, in
                      context, locks, (int)nflags);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  return iris_hip_matmul_all_reduce(A, B, C, aux, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm,
-                                    stride_cn, (const int64_t*)context, 0, 1, block_size_m, block_size_n, block_size_k,
-                                    variant, in_dtype, out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream);
+  return matmul_all_reduce_impl(A, B, C, aux, locks, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm,
+                                stride_cn, (const int64_t*)context, 0, 1, block_size_m, block_size_n, block_size_k,
+                                variant, in_dtype, out_dtype, scale, IRIS_HIP_ACC_FP32, 0, nullptr, path, stream, false, true);
 }
 
 int iris_hip_matmul_reduce_scatter(const void* A, const void* B, void* C, void* aux_buffer, int32_t* locks,
@@ -781,6 +843,8 @@ void iris_hip_debug_set_stamps(void* device_buffer, long long rows) {
   g_stamp_rows = device_buffer ? rows : 0;
 }
 #endif
+
+void iris_hip_set_split_tiles(int32_t mode) { iris_host::set_split_tile_mode(mode); }
 
 const char* iris_hip_last_error(void) { return g_last_error; }
 const char* iris_hip_last_kernel(void) { return g_last_kernel; }

@@ -182,6 +182,114 @@ IRIS_HD int macro_tiles_over_flag_tile(int fm, int fn, int FM, int FN, int KM, i
   return nm * nn;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Tail policy of the 256x256 tile: how the tiles of a partly filled last round are split along K.
+//
+// An XCD's `wgs` workgroups meet `left` (< wgs) tiles in the last round.  Workgroup j < left is the
+// MAIN of tile j: it multiplies the K steps [0, main_steps) and owns the epilogue.  The other
+// wgs - left workgroups are HELPERS that multiply the rest, [main_steps, nsteps), and pass their fp32
+// accumulators on as partial sums:
+//   helpers >= left: every tile gets `per_tile` = helpers / left helpers, each a piece of `piece_steps`
+//                    steps (helper h serves tile h % left with piece 1 + h / left; helpers beyond
+//                    left * per_tile stay idle);
+//   helpers <  left: `per_tile` = 1 and every helper serves `per_helper` = ceil(left / helpers) tiles
+//                    in a row (helper h the tiles h * per_helper ...), one piece [main_steps, nsteps) each.
+// All mains walk K from step 0 at the same pace, as whole tiles of the earlier rounds do, so the operand
+// panels they share keep meeting in the XCD's L2.  (Cutting the round's K steps into equal consecutive
+// shares - the textbook scheme - puts every workgroup at another K offset: measured on 8192 x 1792 x 4096,
+// 224 tiles, the operand traffic from the last-level cache grew ninefold and the launch took 154 us
+// instead of 116.)
+// main_steps balances the main's work (its steps, then `gather_cost` steps' worth of loading each
+// partial sum) against a helper's (per tile: its steps, `pass_cost` steps' worth of pipeline refill and
+// storing the partial sum).  per_tile = 0 means: do not split (nothing to gain).  With both costs at 0
+// (a test setting) every round of at least 4 K steps that can be split is split.
+// ---------------------------------------------------------------------------------------------
+struct SplitPlan {
+  int per_tile;     // helper pieces per tile (0: tiles stay whole)
+  int per_helper;   // tiles a helper serves
+  int main_steps;   // K steps [0, main_steps) stay with the main
+  int piece_steps;  // K steps of a helper piece (the last piece of a tile may be shorter)
+};
+// In K steps of the 256x256 tile (about 0.75 us each), from launches timed with and without the split
+// (bf16, one rank): 16384 x 3584 x 8192 (16 tiles of 32 left) 848 -> 803 us, 8192 x 2880 x 4096 (16 of 32)
+// 197 -> 195, 5120 x 3840 x 4096 (6 of 32, four helpers a tile) 188 -> 186; 4096 x 2880 x 4096 (24 of 32,
+// three tiles a helper) 93 -> 117 and 4096 x 3584 x 8192 (28 of 32) 203 -> 222 when forced, which these
+// costs keep whole.  A 256 KiB partial sum is about 12 us either way: write-through stores at what one CU
+// streams, the flag, a pipeline refill; the flag's round trip and four dependent batches of loads.
+constexpr int kSplitGatherCost = 16;
+constexpr int kSplitPassCost = 16;
+
+IRIS_HD SplitPlan split_plan(int left, int wgs, int nsteps, int gather_cost = kSplitGatherCost, int pass_cost = kSplitPassCost) {
+  SplitPlan s = {0, 1, nsteps, 0};
+  const int helpers = wgs - left;
+  if (left <= 0 || helpers <= 0 || nsteps < 4) return s;
+  int n = 1, m = 1;
+  if (helpers >= left) n = helpers / left; else m = (left + helpers - 1) / helpers;
+  // main_steps + n * gather = m * ((nsteps - main_steps) / n + pass)
+  long num = (long)m * nsteps + (long)n * m * pass_cost - (long)n * n * gather_cost;
+  int main_steps = (int)(num / (n + m));
+  if (main_steps < 1) main_steps = 1;
+  if (main_steps > nsteps - n) return s;        // every helper piece needs a step
+  const int piece = (nsteps - main_steps + n - 1) / n;
+  // The round as its slowest workgroup sees it, in K steps; a split that does not beat a whole tile is none.
+  const int main_cost = main_steps + n * gather_cost;
+  const int helper_cost = m * (piece + pass_cost);
+  if ((main_cost > helper_cost ? main_cost : helper_cost) >= nsteps) return s;
+  s.per_tile = n;
+  s.per_helper = m;
+  s.main_steps = main_steps;
+  s.piece_steps = piece;
+  return s;
+}
+// K steps the slowest workgroup of the round spends, split or not (what the launch code compares).
+IRIS_HD int split_round_steps(const SplitPlan& s, int nsteps, int gather_cost = kSplitGatherCost, int pass_cost = kSplitPassCost) {
+  if (s.per_tile == 0) return nsteps;
+  const int main_cost = s.main_steps + s.per_tile * gather_cost;
+  const int helper_cost = s.per_helper * (s.piece_steps + pass_cost);
+  return main_cost > helper_cost ? main_cost : helper_cost;
+}
+
+// What workgroup `local` (0 .. wgs-1) of an XCD does in the split round as its `served`-th item (0, 1, ...).
+// Returns false when it has nothing (more) to do.  Otherwise tile j (0 .. left-1) of the round, the K
+// steps [k_begin, k_end), and
+//   kind 0: a whole tile (the plan does not split),
+//   kind 1: a helper piece - the accumulators go to partial-sum slot `slot`,
+//   kind 2: the main's piece - the `partners` partial sums in slots slot .. slot + partners - 1 are
+//           added, in that order, before the epilogue.
+// Slots count from 0 within the XCD (all below wgs).  Helpers are the first
+// wgs - left workgroups, mains the last `left`.
+IRIS_HD bool split_item(const SplitPlan& s, int left, int wgs, int nsteps, int local, int served,
+                        int& j, int& k_begin, int& k_end, int& kind, int& partners, int& slot) {
+  const int helpers = wgs - left;
+  k_begin = 0; k_end = nsteps; kind = 0; partners = 0; slot = 0;
+  if (local >= helpers) {  // main
+    if (served > 0) return false;
+    j = local - helpers;
+    if (s.per_tile > 0) {
+      kind = 2;
+      k_end = s.main_steps;
+      const int pieces = (nsteps - s.main_steps + s.piece_steps - 1) / s.piece_steps;
+      partners = pieces < s.per_tile ? pieces : s.per_tile;
+      slot = j * s.per_tile;
+    }
+    return true;
+  }
+  if (s.per_tile == 0 || served >= s.per_helper) return false;
+  int piece = 1;
+  if (s.per_helper > 1) {
+    j = local * s.per_helper + served;
+  } else {
+    j = local % left;
+    piece = 1 + local / left;
+  }
+  k_begin = s.main_steps + (piece - 1) * s.piece_steps;
+  if (j >= left || piece > s.per_tile || k_begin >= nsteps) return false;
+  k_end = k_begin + s.piece_steps < nsteps ? k_begin + s.piece_steps : nsteps;
+  kind = 1;
+  slot = j * s.per_tile + piece - 1;
+  return true;
+}
+
 // The 32x32 small-output kernel addresses A from the operand's first row (of the slot that holds it) and
 // the peers' aux tiles from the buffer's first element, with 32-bit byte offsets into a buffer resource
 // of 2^31 bytes: an offset at or beyond 2^31 would read zeros.  True when every offset the kernel can

@@ -242,6 +242,70 @@ void check_decode_offsets() {
   CHECK(!decode_offsets_fit(0, 512, 512, 2, 64, 64, 64), "no rows");
 }
 
+// The tail policy: for every (tiles left in the last round, workgroups, K steps) the items of all
+// workgroups must cover every K step of every tile exactly once, helpers must come before the mains that
+// wait for them, slots must be distinct and within the XCD's share of the workspace, the main must expect
+// exactly the partial sums that get written, in ascending K order, and the predicted round must never
+// be longer than a whole tile.
+void check_split_plan() {
+  for (int wgs : {4, 32, 38})
+    for (int left = 1; left < wgs; ++left)
+      for (int nsteps : {1, 3, 4, 5, 10, 11, 43, 128, 129, 256, 1000})
+      for (int costs = 0; costs < 2; ++costs) {  // planned with the measured costs, and with none (the test setting)
+        const int gc = costs ? kSplitGatherCost : 0, pc = costs ? kSplitPassCost : 0;
+        const SplitPlan s = split_plan(left, wgs, nsteps, gc, pc);
+        CHECK(split_round_steps(s, nsteps, gc, pc) < nsteps || s.per_tile == 0, "split round not shorter than a tile: %d %d %d", left, wgs, nsteps);
+        std::vector<std::vector<int>> covered(left, std::vector<int>(nsteps, 0));
+        std::vector<int> slot_writer(wgs, -1), slot_begin(wgs, -1);
+        std::vector<int> expects(left, 0), first_slot(left, 0), main_end(left, nsteps);
+        for (int local = 0; local < wgs; ++local)
+          for (int served = 0;; ++served) {
+            int j, kb, ke, kind, partners, slot;
+            if (!split_item(s, left, wgs, nsteps, local, served, j, kb, ke, kind, partners, slot)) break;
+            CHECK(served < 64, "a workgroup never runs out of items");
+            if (served >= 64) break;
+            CHECK(j >= 0 && j < left && kb >= 0 && kb < ke && ke <= nsteps, "item out of range: %d %d %d wg %d", left, wgs, nsteps, local);
+            for (int k = kb; k < ke; ++k) covered[j][k]++;
+            if (kind == 1) {
+              CHECK(local < wgs - left, "helper among the mains");
+              CHECK(slot >= 0 && slot < wgs && slot_writer[slot] < 0, "slot %d reused or out of range (%d %d %d)", slot, left, wgs, nsteps);
+              if (slot >= 0 && slot < wgs) { slot_writer[slot] = j; slot_begin[slot] = kb; }
+            } else {
+              CHECK(local >= wgs - left && kb == 0, "main among the helpers");
+              CHECK((kind == 2) == (s.per_tile > 0), "kind of the main's item");
+              expects[j] = partners; first_slot[j] = slot; main_end[j] = ke;
+            }
+          }
+        for (int j = 0; j < left; ++j) {
+          bool once = true;
+          for (int k = 0; k < nsteps; ++k) once = once && covered[j][k] == 1;
+          CHECK(once, "K steps of tile %d not covered exactly once (%d %d %d)", j, left, wgs, nsteps);
+          int prev = main_end[j];
+          for (int i = 0; i < expects[j]; ++i) {
+            const int sl = first_slot[j] + i;
+            CHECK(sl < wgs && slot_writer[sl] == j && slot_begin[sl] == prev, "main %d expects a partial sum nobody writes (%d %d %d)", j, left, wgs, nsteps);
+            if (sl < wgs && slot_writer[sl] == j) prev = slot_begin[sl] + s.piece_steps;
+          }
+          int written = 0;
+          for (int sl = 0; sl < wgs; ++sl) written += slot_writer[sl] == j;
+          CHECK(written == expects[j], "tile %d: %d partial sums written, %d expected (%d %d %d)", j, written, expects[j], left, wgs, nsteps);
+        }
+      }
+  // worked examples (32 workgroups per XCD).  28 tiles left: 4 helpers would serve 7 tiles each, which
+  // outlasts a whole tile at 128 K steps and gains 4 steps at 256 (the launch code asks for 24); at 1024 it pays
+  CHECK(split_plan(28, 32, 128).per_tile == 0, "28/32/128 stays whole");
+  CHECK(split_round_steps(split_plan(28, 32, 256), 256) == 252, "28/32/256: %d", split_round_steps(split_plan(28, 32, 256), 256));
+  const SplitPlan s = split_plan(28, 32, 1024);
+  CHECK(s.per_tile == 1 && s.per_helper == 7 && s.main_steps == 908 && s.piece_steps == 116, "plan for 28/32/1024: %d %d %d %d", s.per_tile, s.per_helper, s.main_steps, s.piece_steps);
+  CHECK(split_round_steps(s, 1024) == 924, "round of 28/32/1024: %d", split_round_steps(s, 1024));
+  const SplitPlan h = split_plan(16, 32, 256);  // half a round: one helper per tile, equal halves
+  CHECK(h.per_tile == 1 && h.per_helper == 1 && h.main_steps == 128 && h.piece_steps == 128, "plan for 16/32/256: %d %d %d %d", h.per_tile, h.per_helper, h.main_steps, h.piece_steps);
+  CHECK(split_round_steps(h, 256) == 144, "round of 16/32/256");
+  const SplitPlan q = split_plan(6, 32, 256);   // a fifth of a round: four helpers per tile
+  CHECK(q.per_tile == 4 && q.per_helper == 1 && q.main_steps + 4 * q.piece_steps >= 256, "plan for 6/32/256: %d %d %d %d", q.per_tile, q.per_helper, q.main_steps, q.piece_steps);
+  CHECK(split_plan(24, 32, 128).per_tile == 0 || split_round_steps(split_plan(24, 32, 128), 128) > 128 - 24, "24/32/128: too little to gain");
+}
+
 int main() {
   check_row_tile<64>(256);
   check_row_tile<128>(256);
@@ -261,6 +325,7 @@ int main() {
   check_tile_orders();
   check_flag_counts();
   check_decode_offsets();
+  check_split_plan();
   if (failures) { printf("%d check(s) failed\n", failures); return 1; }
   printf("layout_sim: all checks passed\n");
   return 0;
