@@ -345,6 +345,8 @@ WORKLOADS = {
         "matmul_all_reduce_two_shot_bf16_4096x4096x1376", 4096, 4096, 1376, variant="two_shot"),
     "all_gather_matmul_bf16_8192x1792x4096": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096", 8192, 1792, 4096),
     "all_gather_matmul_bf16_8192x1792x4096_nt": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x1792x4096_nt", 8192, 1792, 4096, b_transposed=True),
+    # 32 x 12 = 384 tiles of 256 x 256: one and a half rounds on 256 CUs (the tail policy's case)
+    "all_gather_matmul_bf16_8192x2880x4096": lambda: AllGatherMatmul("all_gather_matmul_bf16_8192x2880x4096", 8192, 2880, 4096),
     "matmul_reduce_scatter_bf16_8192x4096x1376": lambda: MatmulReduceScatter("matmul_reduce_scatter_bf16_8192x4096x1376", 8192, 4096, 1376),
     "matmul_reduce_scatter_accumulate_bf16_8192x4096x1376": lambda: MatmulReduceScatter(
         "matmul_reduce_scatter_accumulate_bf16_8192x4096x1376", 8192, 4096, 1376, accumulate=True),

@@ -292,7 +292,7 @@ int iris_hip_unregister_context(const int64_t* context_tensor);
  * travel through a workspace of the library (64 MiB + 1 KiB per (device, stream), allocated with
  * hipMalloc on the stream's first such launch, never under stream capture - a capturing stream without
  * a workspace launches without splitting -, kept until the process ends, at most 8 per device).
- * mode: -1 the library decides per launch (default: when the split round is expected to be at least 24 K
+ * mode: -1 the library decides per launch (default: when the split round is expected to be at least 16 K
  * steps and an eighth shorter than a whole tile), 0 never split, 1 split whenever the last round is not
  * full and its tiles have at least 4 K steps (a test setting), 2 split whenever any gain is expected (a
  * tuning aid).  The environment variable IRIS_HIP_STREAMK sets the initial mode.  A split launch differs

@@ -155,6 +155,7 @@ __device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, in
   const int nfn = fn_hi - fn_lo + 1;
   const int nft = (fm_hi - fm_lo + 1) * nfn;
   const int items = nft * p.world;
+  bool waited = false;
   for (int i = tid; i < items; i += NT) {
     const int r = i % p.world;
     const int f = i / p.world;
@@ -162,8 +163,11 @@ __device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, in
     const int t = (fm_lo + f / nfn) * ftn + fn_lo + f % nfn;
     if (!p.all_owners && owner_of(p.epi, t, ftotal, p.world, p.rank) != p.rank) continue;
     const int* flag = (const int*)slot_ptr(p.heap_bases, p.locks + t, p.rank, r);
+    // Relaxed system-scope polls (they bypass the caches) and one acquire fence once the flag is up: an
+    // acquire per poll would invalidate the XCD's L2 on every turn of the wait, under the feet of every
+    // workgroup that is still multiplying or storing.
     long long polls = 0;
-    while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != 1) {
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 1) {
       if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
         // A plain system-scope store (one status code, every writer stores the same word): the word
         // may live in pinned host memory.
@@ -172,7 +176,9 @@ __device__ __forceinline__ void wait_peer_flags(const FusedParams& p, int m0, in
       }
       __builtin_amdgcn_s_sleep(8);
     }
+    waited = true;
   }
+  if (waited) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
 }
 
 // One look at the peers' flags that wait_peer_flags would wait for, without waiting: true when
@@ -906,7 +912,10 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 
     if constexpr (STREAMK) {
       // Partial sums travel in the accumulators' own layout: 16-byte piece j of thread t at byte
-      // (j * NT + t) * 16 of the workgroup's slot, so that every wave instruction moves 1 KiB.
+      // (((j + slot) mod PIECES) * NT + t) * 16 of slot `slot`, so that every wave instruction moves 1 KiB.
+      // The rotation by the slot index matters: the slots are 256 KiB apart, and workgroups that store
+      // (or load) piece j at the same moment at the same offset of their slots all meet on a few memory
+      // channels (measured: 20-25 us for the 256 KiB of a slot without it).
       constexpr int PIECES = MB * NB * 4;  // 16-byte pieces per thread
       constexpr long long SLOT_BYTES = (long long)PIECES * NT * 16;
       if (item == ITEM_PART) {
@@ -921,26 +930,31 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           u32x4_t v;
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = __float_as_uint(acc_read(acc.v[mb][nb][4 * q + e]));
-          store16_system_of_valu_data(dst + (long long)j * NT * 16, v);
+          store16_system_of_valu_data(dst + (long long)((j + slot) % PIECES) * NT * 16, v);
           __builtin_amdgcn_sched_barrier(0);  // one piece at a time: the scheduler would read all 128 registers first
         }
         // Published like an aux tile: stores acknowledged by every wave, then one relaxed flag store.
         wait_vmcnt<0>();
         __syncthreads();
         if (tid == 0) __hip_atomic_store(p.sk_flags + slot, p.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        PHASE_STAMP(3);
         continue;  // the ring is free (barrier above); no epilogue for a partial sum
       }
       if (item == ITEM_OWNER) {
         if (tid < partners) {
           const int* flag = p.sk_flags + (slot + tid);
+          // Relaxed polls and one acquire fence at the end: an acquire load per poll would invalidate the
+          // XCD's L2 on every turn while the helpers next door are still storing (measured: their 256 KiB
+          // took 25 us that way).
           long long polls = 0;
-          while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) != p.sk_epoch) {
+          while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != p.sk_epoch) {
             if (p.spin_limit > 0 && ++polls >= p.spin_limit) {
               if (p.status) __hip_atomic_store(p.status, IRIS_HIP_STATUS_SPIN_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
               break;
             }
             __builtin_amdgcn_s_sleep(8);
           }
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
         }
         __syncthreads();
       }
@@ -983,28 +997,24 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       };
       bool staged = false;
       if constexpr (STREAMK) {
-        if (item == ITEM_OWNER) {
-          // own sum + the partners' partial sums in ascending workgroup order, a quarter of the pieces
-          // at a time.  (The accumulators are only read: adding into them in place makes the compiler
+        if (item == ITEM_OWNER && partners > 0) {
+          // own sum + the helper's partial sum, a quarter of the pieces at a time.  (The accumulators are only read: adding into them in place makes the compiler
           // move the whole tile through VGPRs.)
           staged = true;
-          auto slot_of = [&](int pr) -> const char* {
-            unsigned long long base = (unsigned long long)p.sk_partials + (unsigned long long)(slot + pr) * SLOT_BYTES;
-            asm volatile("" : "+s"(base));  // addresses are formed where they are used, not hoisted out of the tile loop
-            return (const char*)base + tid * 16;
-          };
-          auto load_batch = [&](u32x4_t (&dst)[BATCH], const char* src, int b) {
+          unsigned long long base = (unsigned long long)p.sk_partials + (unsigned long long)slot * SLOT_BYTES;
+          asm volatile("" : "+s"(base));  // addresses are formed where they are used, not hoisted out of the tile loop
+          const char* const src = (const char*)base + tid * 16;
+          auto load_batch = [&](u32x4_t (&dst)[BATCH], const char* src, int rot, int b) {  // rot: the slot's index
 #pragma unroll
             for (int i = 0; i < BATCH; ++i)
-              dst[i] = __builtin_nontemporal_load((const u32x4_t*)(src + (long long)(b * BATCH + i) * NT * 16));
+              dst[i] = __builtin_nontemporal_load((const u32x4_t*)(src + (long long)((b * BATCH + i + rot) % PIECES) * NT * 16));
           };
-          if (partners == 1) {  // the usual case: the next batch is on its way while this one is staged
-            const char* const src = slot_of(0);
+          {  // the next batch is on its way while this one is staged
             u32x4_t buf[2][BATCH];
-            load_batch(buf[0], src, 0);
+            load_batch(buf[0], src, slot, 0);
 #pragma unroll
             for (int b = 0; b < NBATCH; ++b) {
-              if (b + 1 < NBATCH) load_batch(buf[(b + 1) & 1], src, b + 1);
+              if (b + 1 < NBATCH) load_batch(buf[(b + 1) & 1], src, slot, b + 1);
 #pragma unroll
               for (int i = 0; i < BATCH; ++i) {
                 float sum[4];
@@ -1014,24 +1024,6 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
                 stage_piece(b * BATCH + i, sum);
               }
               __builtin_amdgcn_sched_barrier(0);
-            }
-          } else {
-#pragma unroll
-            for (int b = 0; b < NBATCH; ++b) {  // unrolled: accumulators are registers, their indices constants
-              float sum[BATCH][4];
-#pragma unroll
-              for (int i = 0; i < BATCH; ++i) own_piece(b * BATCH + i, sum[i]);
-#pragma unroll 1
-              for (int pr = 0; pr < partners; ++pr) {
-                u32x4_t buf[BATCH];
-                load_batch(buf, slot_of(pr), b);
-#pragma unroll
-                for (int i = 0; i < BATCH; ++i)
-#pragma unroll
-                  for (int e = 0; e < 4; ++e) sum[i][e] += __uint_as_float(buf[i][e]);
-              }
-#pragma unroll
-              for (int i = 0; i < BATCH; ++i) stage_piece(b * BATCH + i, sum[i]);
             }
           }
         }
@@ -1342,9 +1334,9 @@ int split_tile_grid(FusedParams& p, int total, int cu_count) {
   const SplitPlan plan = split_plan(left, wg_per_xcd, nsteps, p.sk_gather_cost, p.sk_pass_cost);
   if (plan.per_tile == 0) return 0;
   if (mode == 1 || mode == 2) return grid;  // 2: whatever the plan expects any gain from (a tuning aid)
-  // Worth it when the split round is at least 24 K steps (18 us) and an eighth shorter than a whole tile.
+  // Worth it when the split round is at least 16 K steps (12 us) and an eighth shorter than a whole tile.
   const int steps = split_round_steps(plan, nsteps);
-  return (nsteps - steps >= 24 && (nsteps - steps) * 8 >= nsteps) ? grid : 0;
+  return (nsteps - steps >= 16 && (nsteps - steps) * 8 >= nsteps) ? grid : 0;
 }
 
 template <class CFG>

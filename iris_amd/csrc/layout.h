@@ -185,24 +185,25 @@ IRIS_HD int macro_tiles_over_flag_tile(int fm, int fn, int FM, int FN, int KM, i
 // ---------------------------------------------------------------------------------------------
 // Tail policy of the 256x256 tile: how the tiles of a partly filled last round are split along K.
 //
-// An XCD's `wgs` workgroups meet `left` (< wgs) tiles in the last round.  Workgroup j < left is the
-// MAIN of tile j: it multiplies the K steps [0, main_steps) and owns the epilogue.  The other
-// wgs - left workgroups are HELPERS that multiply the rest, [main_steps, nsteps), and pass their fp32
-// accumulators on as partial sums:
-//   helpers >= left: every tile gets `per_tile` = helpers / left helpers, each a piece of `piece_steps`
-//                    steps (helper h serves tile h % left with piece 1 + h / left; helpers beyond
-//                    left * per_tile stay idle);
-//   helpers <  left: `per_tile` = 1 and every helper serves `per_helper` = ceil(left / helpers) tiles
-//                    in a row (helper h the tiles h * per_helper ...), one piece [main_steps, nsteps) each.
-// All mains walk K from step 0 at the same pace, as whole tiles of the earlier rounds do, so the operand
-// panels they share keep meeting in the XCD's L2.  (Cutting the round's K steps into equal consecutive
-// shares - the textbook scheme - puts every workgroup at another K offset: measured on 8192 x 1792 x 4096,
-// 224 tiles, the operand traffic from the last-level cache grew ninefold and the launch took 154 us
-// instead of 116.)
-// main_steps balances the main's work (its steps, then `gather_cost` steps' worth of loading each
-// partial sum) against a helper's (per tile: its steps, `pass_cost` steps' worth of pipeline refill and
-// storing the partial sum).  per_tile = 0 means: do not split (nothing to gain).  With both costs at 0
-// (a test setting) every round of at least 4 K steps that can be split is split.
+// An XCD's `wgs` workgroups meet `left` (< wgs) tiles in the last round.  When at most half of them
+// would get a tile, workgroup h < left HELPS tile h: the tile's MAIN workgroup (the last `left`
+// workgroups of the XCD) multiplies the K steps [0, main_steps) and owns the epilogue, the helper
+// multiplies [main_steps, nsteps) and passes its fp32 accumulators on as a partial sum.  Helpers beyond
+// `left` stay idle.
+// All mains walk K from step 0 at the same pace and all helpers from main_steps, as the whole tiles of
+// the earlier rounds do, so the operand panels they share keep meeting in the XCD's L2.  What was measured
+// and left out (bf16, one rank, kernel time whole -> split):
+//   - the textbook scheme, the round's K steps cut into equal consecutive shares: every workgroup sits at
+//     another K offset and the operand traffic from the last-level cache grows ninefold
+//     (8192 x 1792 x 4096, 28 of 32 tiles left: 116 -> 154 us);
+//   - several helpers per tile: the main adds their partial sums one after the other
+//     (5120 x 3840 x 4096, 6 of 32 left, four helpers each: 187 -> 192 us; one helper each: 186 -> 163);
+//   - a helper serving several tiles in a row when more than half of the round is filled
+//     (4096 x 2880 x 4096, 24 of 32 left, three tiles per helper: 91 -> 102 us).
+// main_steps balances the main's work (its steps, then `gather_cost` steps' worth of loading the partial
+// sum) against the helper's (its steps, `pass_cost` steps' worth of pipeline fill and storing the partial
+// sum).  per_tile = 0 means: do not split (nothing to gain).  With both costs at 0 (a test setting) every
+// round of at least 4 K steps that can be split is split.
 // ---------------------------------------------------------------------------------------------
 struct SplitPlan {
   int per_tile;     // helper pieces per tile (0: tiles stay whole)
@@ -210,21 +211,19 @@ struct SplitPlan {
   int main_steps;   // K steps [0, main_steps) stay with the main
   int piece_steps;  // K steps of a helper piece (the last piece of a tile may be shorter)
 };
-// In K steps of the 256x256 tile (about 0.75 us each), from launches timed with and without the split
-// (bf16, one rank): 16384 x 3584 x 8192 (16 tiles of 32 left) 848 -> 803 us, 8192 x 2880 x 4096 (16 of 32)
-// 197 -> 195, 5120 x 3840 x 4096 (6 of 32, four helpers a tile) 188 -> 186; 4096 x 2880 x 4096 (24 of 32,
-// three tiles a helper) 93 -> 117 and 4096 x 3584 x 8192 (28 of 32) 203 -> 222 when forced, which these
-// costs keep whole.  A 256 KiB partial sum is about 12 us either way: write-through stores at what one CU
-// streams, the flag, a pipeline refill; the flag's round trip and four dependent batches of loads.
-constexpr int kSplitGatherCost = 16;
-constexpr int kSplitPassCost = 16;
+// In K steps of the 256x256 tile (about 0.75 us each), from time stamps inside a split launch
+// (8192 x 2880 x 4096 bf16): a helper's 256 KiB of partial sums are stored and acknowledged 4.7 us after
+// its last K step, and the next tile's first operands land 3 us later; the main has the partial sum in
+// its staged tile 6 us after the helper's flag went up, 4.5 us more than staging alone takes.
+constexpr int kSplitGatherCost = 8;
+constexpr int kSplitPassCost = 10;
 
 IRIS_HD SplitPlan split_plan(int left, int wgs, int nsteps, int gather_cost = kSplitGatherCost, int pass_cost = kSplitPassCost) {
   SplitPlan s = {0, 1, nsteps, 0};
   const int helpers = wgs - left;
   if (left <= 0 || helpers <= 0 || nsteps < 4) return s;
-  int n = 1, m = 1;
-  if (helpers >= left) n = helpers / left; else m = (left + helpers - 1) / helpers;
+  if (helpers < left) return s;  // more than half of the round is filled
+  const int n = 1, m = 1;
   // main_steps + n * gather = m * ((nsteps - main_steps) / n + pass)
   long num = (long)m * nsteps + (long)n * m * pass_cost - (long)n * n * gather_cost;
   int main_steps = (int)(num / (n + m));
@@ -254,8 +253,7 @@ IRIS_HD int split_round_steps(const SplitPlan& s, int nsteps, int gather_cost = 
 // steps [k_begin, k_end), and
 //   kind 0: a whole tile (the plan does not split),
 //   kind 1: a helper piece - the accumulators go to partial-sum slot `slot`,
-//   kind 2: the main's piece - the `partners` partial sums in slots slot .. slot + partners - 1 are
-//           added, in that order, before the epilogue.
+//   kind 2: the main's piece - the partial sum in slot `slot` is added before the epilogue (partners = 1).
 // Slots count from 0 within the XCD (all below wgs).  Helpers are the first
 // wgs - left workgroups, mains the last `left`.
 IRIS_HD bool split_item(const SplitPlan& s, int left, int wgs, int nsteps, int local, int served,

@@ -291,19 +291,15 @@ void check_split_plan() {
           CHECK(written == expects[j], "tile %d: %d partial sums written, %d expected (%d %d %d)", j, written, expects[j], left, wgs, nsteps);
         }
       }
-  // worked examples (32 workgroups per XCD).  28 tiles left: 4 helpers would serve 7 tiles each, which
-  // outlasts a whole tile at 128 K steps and gains 4 steps at 256 (the launch code asks for 24); at 1024 it pays
-  CHECK(split_plan(28, 32, 128).per_tile == 0, "28/32/128 stays whole");
-  CHECK(split_round_steps(split_plan(28, 32, 256), 256) == 252, "28/32/256: %d", split_round_steps(split_plan(28, 32, 256), 256));
-  const SplitPlan s = split_plan(28, 32, 1024);
-  CHECK(s.per_tile == 1 && s.per_helper == 7 && s.main_steps == 908 && s.piece_steps == 116, "plan for 28/32/1024: %d %d %d %d", s.per_tile, s.per_helper, s.main_steps, s.piece_steps);
-  CHECK(split_round_steps(s, 1024) == 924, "round of 28/32/1024: %d", split_round_steps(s, 1024));
-  const SplitPlan h = split_plan(16, 32, 256);  // half a round: one helper per tile, equal halves
-  CHECK(h.per_tile == 1 && h.per_helper == 1 && h.main_steps == 128 && h.piece_steps == 128, "plan for 16/32/256: %d %d %d %d", h.per_tile, h.per_helper, h.main_steps, h.piece_steps);
-  CHECK(split_round_steps(h, 256) == 144, "round of 16/32/256");
-  const SplitPlan q = split_plan(6, 32, 256);   // a fifth of a round: four helpers per tile
-  CHECK(q.per_tile == 4 && q.per_helper == 1 && q.main_steps + 4 * q.piece_steps >= 256, "plan for 6/32/256: %d %d %d %d", q.per_tile, q.per_helper, q.main_steps, q.piece_steps);
-  CHECK(split_plan(24, 32, 128).per_tile == 0 || split_round_steps(split_plan(24, 32, 128), 128) > 128 - 24, "24/32/128: too little to gain");
+  // worked examples (32 workgroups per XCD).  More than half of the round filled: the tiles stay whole
+  CHECK(split_plan(28, 32, 128).per_tile == 0 && split_plan(28, 32, 1024).per_tile == 0 && split_plan(17, 32, 1024).per_tile == 0,
+        "a round that is more than half full stays whole");
+  const SplitPlan h = split_plan(16, 32, 256);  // half a round: one helper per tile, about equal halves
+  CHECK(h.per_tile == 1 && h.per_helper == 1 && h.main_steps == 129 && h.piece_steps == 127, "plan for 16/32/256: %d %d %d %d", h.per_tile, h.per_helper, h.main_steps, h.piece_steps);
+  CHECK(split_round_steps(h, 256) == 137, "round of 16/32/256");
+  const SplitPlan q = split_plan(6, 32, 256);   // a fifth of a round: still one helper per tile, twenty stay idle
+  CHECK(q.per_tile == 1 && q.per_helper == 1 && q.main_steps == h.main_steps, "plan for 6/32/256: %d %d %d %d", q.per_tile, q.per_helper, q.main_steps, q.piece_steps);
+  CHECK(split_plan(16, 32, 16).per_tile == 0, "16 K steps: the partial sum costs more than it saves");
 }
 
 int main() {

@@ -1,8 +1,8 @@
-"""GPU parity tests of the tail policy of the 256x256 tile: in a last round of tiles that is partly
-empty, the workgroups without a tile multiply pieces of the others' K ranges and pass fp32 partial sums
-on.  Integer-valued inputs make every partial sum exact, so the split launch must give the oracle's bits
-wherever the split points are; the shapes put them next to K tails, across the source slots of a gathered
-A, give a tile one helper or four, and a helper one tile or several."""
+"""GPU parity tests of the tail policy of the 256x256 tile: in a last round of tiles that is at most half
+full, workgroups without a tile multiply the second part of the others' K ranges and pass fp32 partial
+sums on.  Integer-valued inputs make every partial sum exact, so the split launch must give the oracle's
+bits wherever the split point is; the shapes put it next to K tails and between the source slots of a
+gathered A, after one whole round of tiles."""
 
 import pytest
 import torch
@@ -26,13 +26,12 @@ def _ctx(world, rank=0, heap=1 << 28):
     return iris.iris(heap, num_ranks=world, rank=rank)
 
 
-# tiles of 256 x 256 on 256 CUs in 8 XCDs (32 workgroups each):
-#   3584 x 3072 = 14 x 12 = 168 tiles: 21 per XCD, no full round: 11 helpers serve two tiles each
-#   5120 x 3840 = 20 x 15 = 300 tiles: 38 per XCD (34 in the last): one full round, then 6 (2) tiles with
-#                                      four (fifteen) helpers each
-#   2304 x 4096 =  9 x 16 = 144 tiles: 18 per XCD, 14 helpers
+# tiles of 256 x 256 on 256 CUs in 8 XCDs (32 workgroups each); every XCD first takes a whole round of 32:
+#   5120 x 3840 = 20 x 15 = 300 tiles: 38 per XCD (34 in the last XCD): 6 (2) tiles left for the split round
+#   5120 x 4096 = 20 x 16 = 320 tiles: 40 per XCD: 8 left
+#   4352 x 4096 = 17 x 16 = 272 tiles: 34 per XCD: 2 left
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float8_e4m3fn], ids=["bf16", "f16", "fp8"])
-@pytest.mark.parametrize("M,N,K", [(3584, 3072, 320), (5120, 3840, 512), (2304, 4096, 1040), (3584, 3072, 272)])
+@pytest.mark.parametrize("M,N,K", [(5120, 3840, 320), (5120, 4096, 512), (4352, 4096, 1040), (5120, 3840, 272)])
 def test_plain_gemm_split(dtype, M, N, K):
     """all_gather_matmul with one rank is the plain GEMM; K = 1040 and 272 end in a partial K step."""
     fp8 = dtype == torch.float8_e4m3fn
@@ -56,12 +55,12 @@ def test_gathered_a_split(gather_dim, W, rank):
     dtype = torch.bfloat16
     ctx = _ctx(W, rank)
     if gather_dim == 1:
-        M, N, Kl = 3584, 3072, 80
+        M, N, Kl = 5120, 3840, 80
         shards = [randint_cpu((M, Kl), 10 + r, dtype) for r in range(W)]
         B = randint_cpu((W * Kl, N), 30, dtype)
         rows = M
     else:
-        M_local, N, Kl = 512, 2816, 200  # 4096 x 2816 = 16 x 11 = 176 tiles: 22 per XCD, 10 helpers with three tiles each
+        M_local, N, Kl = 768, 3328, 200  # 6144 x 3328 = 24 x 13 = 312 tiles: 39 per XCD, 7 left
         shards = [randint_cpu((M_local, Kl), 10 + r, dtype) for r in range(W)]
         B = randint_cpu((Kl, N), 30, dtype)
         rows = W * M_local
@@ -77,12 +76,12 @@ def test_gathered_a_split(gather_dim, W, rank):
     assert_bits_equal(out.cpu(), oracle.all_gather_matmul(shards, B, bias=bias, gather_dim=gather_dim), kernel)
 
 
-@pytest.mark.parametrize("variant,M,N,K", [("one_shot", 3584, 3072, 200), ("one_shot", 5120, 3840, 192), ("two_shot", 3584, 3072, 200)])
-def test_all_reduce_split(variant, M, N, K):
-    """The owner of a split tile runs the whole epilogue: aux, flags, the slot sum over the peers.  (A
-    two-shot launch with more tiles than CUs keeps one workgroup per tile and is not split.)  K = 192 is
-    six K steps for a main and four helpers: one step, three pieces of two and one, and a helper left over."""
-    W, rank, dtype = 4, 1, torch.bfloat16
+@pytest.mark.parametrize("variant,W,rank,M,N,K", [("one_shot", 4, 1, 5120, 3840, 200), ("one_shot", 2, 0, 5120, 4096, 192),
+                                                  ("two_shot", 1, 0, 5120, 3840, 200)])
+def test_all_reduce_split(variant, W, rank, M, N, K):
+    """The main of a split tile runs the whole epilogue: aux, flags, the slot sum over the peers.  (A
+    two-shot launch with peers and more tiles than CUs keeps one workgroup per tile and is not split.)"""
+    dtype = torch.bfloat16
     ctx = _ctx(W, rank, heap=1 << 29)
     A, B = randint_cpu((M, K), 5, dtype), randint_cpu((K, N), 6, dtype)
     peers = [randn_cpu((M, N), 40 + r, dtype) for r in range(W)]
@@ -105,7 +104,7 @@ def test_all_reduce_split(variant, M, N, K):
 def test_split_launches_in_a_row_and_on_two_streams():
     """The flags of the workspace are never cleared: every launch uses a new flag value.  Three launches in
     a row on one stream, then one on a second stream (which gets a workspace of its own), each checked."""
-    dtype, M, N, K = torch.bfloat16, 3584, 3072, 136
+    dtype, M, N, K = torch.bfloat16, 5120, 3840, 136
     ctx = _ctx(1)
     outs = []
     side = torch.cuda.Stream()
@@ -129,10 +128,10 @@ def test_split_launches_in_a_row_and_on_two_streams():
 
 def test_random_data_within_tolerance_and_default_rule():
     """Random data: the split launch sums K in another order, the result stays within the bf16 bound.  And
-    the default rule: a short K loop is not split, a long one with a partly empty round is."""
-    dtype, M, N = torch.bfloat16, 3584, 3072
-    ctx = _ctx(1)
-    for K, want_split in ((256, False), (8192, True)):
+    the default rule: a short K loop is not split, a long one with a last round that is a fifth full is."""
+    dtype, M, N = torch.bfloat16, 5120, 3840
+    ctx = _ctx(1, heap=1 << 29)
+    for K, want_split in ((256, False), (4096, True)):
         A, B = randn_cpu((M, K), 90, dtype, K ** -0.5), randn_cpu((K, N), 91, dtype, K ** -0.5)
         dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
         out = ctx.zeros((M, N), dtype=dtype)
