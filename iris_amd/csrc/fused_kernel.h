@@ -238,14 +238,24 @@ struct MfmaCfg {
   static constexpr int LA = A_BYTES / kDmaBytes / NW;  // direct-to-LDS loads per thread per K step
   static constexpr int LB = B_BYTES / kDmaBytes / NW;
   static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
-  // Epilogue staging: the whole output tile in 16-bit elements, rows padded by 16 bytes so that
-  // the accumulator-layout writes (one row per lane) spread over the LDS banks.
-  static constexpr int TROW = BN * 2 + 16;
+  // Epilogue staging: the whole output tile in 16-bit elements.  The accumulator-layout writes put one
+  // row per lane, so rows must not start on the same LDS banks.  The four-wave tiles pad every row by 16
+  // bytes and stage over the (dead) operand ring from its start.  The eight-wave tile has no LDS to
+  // spare for padding: it XORs the 16-byte chunk index with the row instead, and stages above the first
+  // ring slot, which leaves that slot free to take the first K step of the workgroup's NEXT tile while
+  // this tile's epilogue is still streaming (160 KiB = one ring slot + the staged tile).
+  static constexpr bool STAGE_SWIZZLED = (NW == 8);
+  static constexpr int STAGE_OFF = STAGE_SWIZZLED ? STAGE_BYTES : 0;
+  static constexpr int TROW = STAGE_SWIZZLED ? BN * 2 : BN * 2 + 16;
   static constexpr int TILE_BYTES = BM * TROW;
-  // One word per wave behind the staged tile, for workgroup-wide votes in the epilogue (workgroup_all).
-  static constexpr int VOTE_OFFSET = TILE_BYTES;
-  static constexpr int SMEM_BYTES = RING_BYTES > TILE_BYTES + 64 ? RING_BYTES : TILE_BYTES + 64;
+  static constexpr int SMEM_BYTES = RING_BYTES > STAGE_OFF + TILE_BYTES ? RING_BYTES : STAGE_OFF + TILE_BYTES;
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+  static_assert(!STAGE_SWIZZLED || ((BN / 8) & (BN / 8 - 1)) == 0, "chunk swizzle needs a power-of-two row");
+  // LDS byte offset of byte `b` of row `row` of the staged tile.
+  __host__ __device__ static constexpr int stage_offset(int row, int b) {
+    if (STAGE_SWIZZLED) return STAGE_OFF + row * TROW + ((((b >> 4) ^ row) & (BN / 8 - 1)) << 4) + (b & 15);
+    return row * TROW + b;
+  }
   // Four-wave tiles whose ring fits twice into a CU's LDS run two workgroups per CU, so that the
   // memory round trips of one workgroup's epilogue hide behind the other's K loop.
   static constexpr int WG_PER_CU = (NW == 4 && SMEM_BYTES <= 80 * 1024) ? 2 : 1;
@@ -332,22 +342,6 @@ __device__ __forceinline__ float acc_add(float a, float x) {
 
 __device__ __forceinline__ unsigned lds_address(const void* p) {
   return (unsigned)(unsigned long long)(LDS_AS const char*)p;
-}
-
-// True when `pred` holds in every thread of the workgroup; doubles as a workgroup barrier (two of them).
-// The votes of the waves meet in `words` (one int per wave, LDS that nothing else uses at this point).
-// Unlike __syncthreads_and it takes no static LDS of its own, which would come on top of the dynamic
-// LDS and so cap the operand ring one KiB short of the CU's 160 KiB.
-template <int NW>
-__device__ __forceinline__ bool workgroup_all(bool pred, char* words, int wave, int lane) {
-  const int mine = __all(pred) ? 1 : 0;
-  if (lane == 0) *(LDS_AS int*)(LDS_AS char*)(words + 4 * wave) = mine;
-  __syncthreads();
-  int all = 1;
-#pragma unroll
-  for (int w = 0; w < NW; ++w) all &= *(const LDS_AS int*)(LDS_AS char*)(words + 4 * w);
-  __syncthreads();  // the words may be rewritten (next tile's vote) only after everybody has read them
-  return all != 0;
 }
 
 template <class CFG>
@@ -628,6 +622,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     plan = split_plan(sk_left, wg_per_xcd, nsteps, p.sk_gather_cost, p.sk_pass_cost);
   }
 
+  // Looping workgroups of the eight-wave tile fetch the first K step of their next tile into ring slot 0
+  // as soon as the K loop of the current tile is over (the staged tile lives above that slot): the loads
+  // go out ahead of the epilogue's stores instead of behind them, and their latency - cold operand panels,
+  // 2-3 us - passes under the epilogue.
+  constexpr bool PREFETCH_NEXT = CFG::STAGE_SWIZZLED && !ONE_ROUND && !STREAMK;
+  bool first_step_prefetched = false;
+
   for (int it = 0; ONE_ROUND ? it < 1 : true; ++it) {
     int tidx, k_begin = 0, k_end = nsteps, item = ITEM_WHOLE, partners = 0, slot = 0;
     if constexpr (STREAMK) {
@@ -739,7 +740,13 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     // single-group loop, so it keeps one step less in flight.
     constexpr int AHEAD = PINGPONG ? STAGES - 2 : STAGES - 1;  // K steps issued before the loop starts
 #pragma unroll
-    for (int s = 0; s < AHEAD; ++s) issue(s);
+    for (int s = 0; s < AHEAD; ++s) {
+      if (PREFETCH_NEXT && s == 0 && first_step_prefetched)
+        end_step();  // already on its way (or there): only the loader position moves on
+      else
+        issue(s);
+    }
+    first_step_prefetched = false;
     wait_vmcnt<(AHEAD - 1) * (LA + LB)>();
     __builtin_amdgcn_s_barrier();
     PHASE_STAMP(1);
@@ -960,6 +967,36 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       }
     }
 
+    if constexpr (PREFETCH_NEXT) {
+      const int nidx = xcd_tile_index(blockIdx.x, gridDim.x, it + 1, total_tiles, p.num_xcd);
+      if (nidx >= 0) {
+        int ntm, ntn;
+        grouped_tile(nidx, p.tiles_m, p.tiles_n, p.group_m, ntm, ntn);
+        const int nm0 = ntm * BM, nn0 = ntn * BN;
+        int n_slot = p.rank;
+        long long n_row0 = nm0;
+        if (p.gather == GATHER_M) {
+          n_slot = nm0 / p.M_local;
+          n_row0 = nm0 - (long long)n_slot * p.M_local;
+        }
+        if (p.gather == GATHER_K) n_slot = 0;
+        const i32x4_t nra = make_rsrc_words((p.gather == GATHER_NONE ? a_own : in_slot(a_own, n_slot)) + (unsigned long long)(n_row0 * p.s_am * ES));
+        const i32x4_t nrb = make_rsrc_words((unsigned long long)p.B + (unsigned long long)nn0 * (CFG::B_KCONTIG ? p.s_bn : 1) * ES);
+        const unsigned sa = smem_base + wave * kDmaBytes, sb = sa + CFG::A_BYTES;  // ring slot 0
+#pragma unroll
+        for (int j = 0; j < LA; ++j) {
+          const bool ok = nm0 + la_row[j] < p.M && la_k[j] < klocal;
+          dma16(nra, sa + j * NW * kDmaBytes, ok ? la_off[j] : kInvalidOffset, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+          const bool ok = CFG::B_KCONTIG ? (nn0 + lb_row[i] < p.N && lb_col[i] < klocal) : (nn0 + lb_col[i] < p.N && lb_row[i] < klocal);
+          dma16(nrb, sb + i * NW * kDmaBytes, ok ? lb_off[i] : kInvalidOffset, 0u);
+        }
+        first_step_prefetched = true;
+      }
+    }
+
     // ---- epilogue -------------------------------------------------------------------------------
     // The whole output tile is first written to LDS in the output type (the operand ring is dead
     // by now), which frees the accumulators; both phases then stream rows of the tile, 16 bytes per
@@ -977,6 +1014,11 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           if (gm < p.M) badd[mb] = load_scalar_as_float(p.bias, (long long)gm * p.s_bias, p.bias_dtype);
         }
       }
+      // The lane index as the staging addresses see it goes through an empty asm: with the swizzled layout
+      // a lane has one address term per (column block, quarter), and the compiler would otherwise compute
+      // them once, ahead of the tile loop, and carry eight more registers through the K loop.
+      int lane_s = lane;
+      asm volatile("" : "+v"(lane_s));
       // Piece j of the thread: 4 consecutive n of one m, from their fp32 sums to the staged tile.
       auto stage_piece = [&](int j, const float (&sum)[4]) {
         const int mb = j / (NB * 4), nb = (j / 4) % NB, q = j % 4;
@@ -986,9 +1028,9 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         u32x2_t w;
         w.x = Out::pack(h[0], h[1]);
         w.y = Out::pack(h[2], h[3]);
-        const int trow = wm * TM + mb * 32 + acc_col(lane);
-        const int tcol = wn * TN + nb * 32 + acc_row(lane, 4 * q);
-        *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + trow * CFG::TROW + tcol * 2) = w;
+        const int trow = wm * TM + mb * 32 + acc_col(lane_s);
+        const int tcol = wn * TN + nb * 32 + acc_row(lane_s, 4 * q);
+        *(LDS_AS u32x2_t*)(LDS_AS char*)(smem + CFG::stage_offset(trow, tcol * 2)) = w;
       };
       auto own_piece = [&](int j, float (&sum)[4]) {
         const int mb = j / (NB * 4), nb = (j / 4) % NB, q = j % 4;
@@ -1043,10 +1085,15 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     constexpr int CPR = BN / 8;            // 16-byte chunks per tile row
     constexpr int RPP = NT / CPR;          // tile rows covered by one pass of the workgroup
     constexpr int PASSES = BM / RPP;
-    const int t_row = tid / CPR, t_chunk = tid % CPR;
+    int tid_s = tid;  // as lane_s above: per-thread staging offsets are formed here, not ahead of the tile loop
+    asm volatile("" : "+v"(tid_s));
+    const int t_row = tid_s / CPR, t_chunk = tid_s % CPR;
     const int gn = n0 + t_chunk * 8;
     const bool col_ok = gn < p.N;
-    const char* const t_lds = smem + t_row * CFG::TROW + t_chunk * 16;
+    // LDS offset of this thread's chunk in pass ps: t_pass[ps & 1] + ps * RPP * TROW (the passes are RPP
+    // rows apart; with the swizzled layout the chunk's place in the row alternates between two values).
+    static_assert(!CFG::STAGE_SWIZZLED || (2 * RPP) % CPR == 0, "the swizzle must repeat every two passes");
+    const int t_pass[2] = {CFG::stage_offset(t_row, t_chunk * 16), CFG::stage_offset(t_row + RPP, t_chunk * 16) - RPP * CFG::TROW};
 
     // Phase 1: C (plain store) or aux (own slot).  When no peer contributes (world of one, or peers
     // switched off) the reduced tile equals the own tile, so C is written in the same pass and
@@ -1073,7 +1120,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
             const int row = ps * RPP + d / DPR, dc = d % DPR;
             const int gm = m0 + row, gc = n0 + 2 * dc;
             if (gm >= p.M || gc >= p.N) continue;
-            const unsigned w = *(const LDS_AS unsigned*)(LDS_AS char*)(smem + row * CFG::TROW + dc * 4);
+            const unsigned w = *(const LDS_AS unsigned*)(LDS_AS char*)(smem + CFG::stage_offset(row, dc * 4));
             const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gc) * 2;
             for (int pr = 0; pr < p.world; ++pr) atomic_add_packed<Out>((char*)(in_slot(c_base, pr) + eoff), w);
           }
@@ -1082,7 +1129,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 #pragma unroll 4
       for (int ps = 0; ps < PASSES; ++ps) {
         const int gm = m0 + ps * RPP + t_row;
-        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(t_lds + ps * RPP * CFG::TROW);
+        const u32x4_t v = *(const LDS_AS u32x4_t*)(LDS_AS char*)(smem + t_pass[ps & 1] + ps * RPP * CFG::TROW);
         if (gm < p.M && col_ok) {
           const long long eoff = ((long long)(gm + p.row_offset) * p.s_cm + gn) * 2;
           if (p.epi == EPI_ALL_GATHER) {
@@ -1116,19 +1163,18 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
       // (no L2 write-back is needed any more).  Likewise the peers' flags are polled (system-scope
       // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
       // every wave poll and run ahead measured slower.
-      // The peers' flags are looked at once while the own stores are still on their way: when all of
-      // them are up already - peers that finished first - their round trip hides behind that wait
-      // and the polling after the own flags are raised is skipped.
+      // The peers' flags are looked at once while the own stores are still on their way: a thread that
+      // found the flags it is responsible for up already - peers that finished first - has their round
+      // trip hidden behind that wait and does not poll after the own flags are raised.  Every thread
+      // knows only about its own flags; the barrier behind the polling makes it common knowledge.
       const bool up_already = solo ? true : probe_peer_flags<BM, BN, NT>(p, m0, n0, tid);
       wait_vmcnt<0>();
-      const bool all_up = workgroup_all<NW>(up_already, smem + CFG::VOTE_OFFSET, wave, lane);
+      __syncthreads();
       PHASE_STAMP(5);
       raise_flags<BM, BN, NT, true>(p, m0, n0, tid);
       if (!solo) {
-        if (!all_up) {
-          wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
-          __syncthreads();
-        }
+        if (!up_already) wait_peer_flags<BM, BN, NT>(p, m0, n0, tid);
+        __syncthreads();
       }
       PHASE_STAMP(6);
 
@@ -1183,7 +1229,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
               gc = c0 + (int)(idx - row * (unsigned)ncw) * 8;
               owner[g] = rect_owner;
               active[g] = gm < r1;
-              lds_off = active[g] ? (gm - m0) * CFG::TROW + (gc - n0) * 2 : 0;
+              lds_off = active[g] ? CFG::stage_offset(gm - m0, (gc - n0) * 2) : CFG::stage_offset(0, 0);
             } else {
               gm = m0 + (pg + g) * RPP + t_row;
               gc = gn;
@@ -1193,7 +1239,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
                 owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
               }
               active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
-              lds_off = ((pg + g) * RPP + t_row) * CFG::TROW + t_chunk * 16;
+              lds_off = t_pass[(pg + g) & 1] + (pg + g) * RPP * CFG::TROW;
             }
             eoff[g] = active[g] ? ((long long)gm * p.s_cm + gc) * 2 : safe_off;
             if constexpr (NP > 0) {
