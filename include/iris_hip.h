@@ -290,8 +290,9 @@ int iris_hip_unregister_context(const int64_t* context_tensor);
  * workgroups partly empty for many K steps, the K steps of that round's tiles are shared out evenly
  * between all workgroups; a tile that ends up in several shares is summed from fp32 partial sums that
  * travel through a workspace of the library (64 MiB + 1 KiB per (device, stream), allocated with
- * hipMalloc on the stream's first such launch, never under stream capture - a capturing stream without
- * a workspace launches without splitting -, kept until the process ends, at most 8 per device).
+ * hipMalloc on the stream's first such launch, kept until the process ends, at most 8 per device).
+ * Launches on a capturing stream are never split: the flag value that tells this launch's partial sums
+ * from the previous launch's is a kernel argument and would repeat on every replay.
  * mode: -1 the library decides per launch (default: when the split round is expected to be at least 16 K
  * steps and an eighth shorter than a whole tile), 0 never split, 1 split whenever the last round is not
  * full and its tiles have at least 4 K steps (a test setting), 2 split whenever any gain is expected (a

@@ -16,7 +16,7 @@ int device_facts(int device, int* cu_count, int* xcc_count);
 // sums, `nwg` flags, and the value the flags take in this launch.  One workspace per (device, stream),
 // allocated on the stream's first such launch and kept until the process ends; launches on one stream
 // are ordered, so they can share it.  Returns 0, or non-zero when there is none to be had (the stream is
-// being captured and has no workspace yet, a device's eight workspaces are taken, the allocation failed):
+// being captured, a device's eight workspaces are taken, the allocation failed):
 // the caller then launches without splitting tiles.
 // -1 decide per launch, 0 never split tiles, 1 split whenever the last round of tiles is not full.
 int split_tile_mode();

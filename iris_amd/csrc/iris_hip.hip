@@ -580,6 +580,14 @@ int split_tile_mode() { return g_split_mode.load(std::memory_order_relaxed); }
 void set_split_tile_mode(int mode) { g_split_mode.store(mode < 0 ? -1 : (mode > 2 ? 2 : mode), std::memory_order_relaxed); }
 
 int split_tile_workspace(int device, hipStream_t stream, int nwg, long long slot_bytes, char** partials, int** flags, int* epoch) {
+  // Never under stream capture: the flag value of a launch is a kernel argument, a replayed launch would
+  // meet the flags of its previous replay already at that value and read partial sums before they are
+  // written.  (And nothing may be allocated or cleared on a capturing stream.)
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return 1;
+  }
   std::lock_guard<std::mutex> lock(g_split_mutex);
   int on_device = 0;
   for (SplitTileWorkspace& w : g_split_workspaces) {
@@ -593,12 +601,7 @@ int split_tile_workspace(int device, hipStream_t stream, int nwg, long long slot
     return 0;
   }
   if (on_device >= kMaxSplitWorkspacesPerDevice) return 1;
-  // First split launch on this stream.  Nothing may be allocated or cleared on a stream under capture.
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return 1;
-  }
+  // First split launch on this stream.
   SplitTileWorkspace w{device, stream, nullptr, nullptr, nwg, slot_bytes, 1u};
   if (hipMalloc((void**)&w.partials, (size_t)nwg * (size_t)slot_bytes) != hipSuccess) {
     (void)hipGetLastError();

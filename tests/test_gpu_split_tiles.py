@@ -126,6 +126,35 @@ def test_split_launches_in_a_row_and_on_two_streams():
         assert_bits_equal(out.cpu(), want, f"launch {i}")
 
 
+def test_captured_launches_are_not_split():
+    """A launch recorded into a HIP graph keeps its tiles whole (its flag value would repeat on every
+    replay); the replays give the oracle's bits, with eager split launches in between."""
+    dtype, M, N, K = torch.bfloat16, 5120, 3840, 136
+    ctx = _ctx(1)
+    A, B = randint_cpu((M, K), 95, dtype), randint_cpu((K, N), 96, dtype)
+    dA, dB = heap_tensor(ctx, A), heap_tensor(ctx, B)
+    out, eager = ctx.zeros((M, N), dtype=dtype), ctx.zeros((M, N), dtype=dtype)
+    want = oracle.all_gather_matmul([A], B)
+    ops.all_gather_matmul(ctx, eager, dA, dB)  # the stream has a workspace by now
+    assert _lib.last_kernel().endswith("_splitk")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ops.all_gather_matmul(ctx, out, dA, dB, async_op=True)
+    assert not _lib.last_kernel().endswith("_splitk"), _lib.last_kernel()
+    for replay in range(3):
+        out.zero_()
+        eager.zero_()
+        ops.all_gather_matmul(ctx, eager, dA, dB)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(out.cpu(), want, f"replay {replay}")
+        assert_bits_equal(eager.cpu(), want, f"eager launch before replay {replay}")
+
+
 def test_random_data_within_tolerance_and_default_rule():
     """Random data: the split launch sums K in another order, the result stays within the bf16 bound.  And
     the default rule: a short K loop is not split, a long one with a last round that is a fifth full is."""
