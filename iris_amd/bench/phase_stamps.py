@@ -34,6 +34,10 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--dump", default=None, metavar="FILE.npy",
                     help="save the last launch's stamps (microseconds, one row of 9 per tile) for other tools")
+    ap.add_argument("--items", type=int, default=0, metavar="GRID",
+                    help="also print, for the last launch of GRID workgroups, the mean stamps of every workgroup's first, "
+                         "second, ... tile separately (split launches: helpers' pieces end at stamp 3, 'partial sum out')")
+    ap.add_argument("--split", type=int, default=None, metavar="MODE", help="iris_hip_set_split_tiles(MODE) before the launches")
     ap.add_argument("--deciles", action="store_true",
                     help="also print, for the last launch, the deciles over the stamped tiles of every phase")
     args = ap.parse_args()
@@ -57,6 +61,8 @@ def main():
     hip.gpu_try(hip.runtime().hipDeviceGetAttribute(ctypes.byref(rate_khz), 10017, 0))  # hipDeviceAttributeWallClockRate
     us_per_tick = 1e3 / rate_khz.value
 
+    if args.split is not None:
+        lib.iris_hip_set_split_tiles(args.split)
     wl = bench.WORKLOADS[args.workload or bench.DEFAULT]()
     wl.setup(iris, args.world)
     max_wgs = 65536  # rows of the stamp buffer: tiles stamped per launch (eight per workgroup at most)
@@ -80,6 +86,7 @@ def main():
         if rep < 0:
             continue
         t = stamps.cpu()
+        raw = t.double() * us_per_tick
         t = t[t[:, 0] != 0].double() * us_per_tick
         last = 8
         while last > 0 and float(t[:, last].max()) == 0.0:  # phases this launch does not have
@@ -93,9 +100,11 @@ def main():
                 per_phase[i].append(0.0)
                 per_phase_max[i].append(0.0)
                 continue
-            per_phase[i].append(float((cur - prev).mean()))
-            per_phase_max[i].append(float((cur - prev).max()))
-            prev = cur
+            both = (cur != 0) & (prev != 0)  # helpers' pieces of a split launch stop at stamp 3
+            d = (cur - prev)[both]
+            per_phase[i].append(float(d.mean()) if d.numel() else 0.0)
+            per_phase_max[i].append(float(d.max()) if d.numel() else 0.0)
+            prev = torch.where(cur != 0, cur, prev)
         spans.append(float(t[:, last].max()) - t0)
     print(f"workload {wl.name}  W={args.world}  kernel {_lib.last_kernel()}  tiles stamped {t.shape[0]}  flush={args.flush}  "
           f"{args.reps} launches; microseconds, mean over launches of (mean | max over tiles)")
@@ -103,6 +112,20 @@ def main():
     for name, mean, mx in zip(PHASES, per_phase, per_phase_max):
         print(f"  {name:40s} {statistics.mean(mean):8.2f} | {statistics.mean(mx):8.2f}")
     print(f"  {'first entry -> last stamp':40s} {statistics.mean(spans):8.2f}")
+    if args.items:
+        grid = args.items
+        print(f"  last launch, per workgroup item (rows item * {grid} + workgroup), mean stamp in us after the first entry:")
+        print("    item   rows  " + " ".join(f"{i:>7d}" for i in range(9)))
+        for item in range(8):
+            rows = raw[item * grid:(item + 1) * grid]
+            if not bool((rows[:, 0] != 0).any()):
+                continue
+            for name, part in (("workgroups of the first half of the grid", rows[: grid // 2]), ("second half", rows[grid // 2:])):
+                part = part[part[:, 0] != 0]
+                if part.shape[0] == 0:
+                    continue
+                cols = [f"{float((part[:, i][part[:, i] != 0] - t0).mean()):7.1f}" if bool((part[:, i] != 0).any()) else "      -" for i in range(9)]
+                print(f"    {item:4d} {part.shape[0]:6d}  " + " ".join(cols) + f"   ({name})")
     if args.dump:
         import numpy
         os.makedirs(os.path.dirname(os.path.abspath(args.dump)), exist_ok=True)
