@@ -919,10 +919,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
 
     if constexpr (STREAMK) {
       // Partial sums travel in the accumulators' own layout: 16-byte piece j of thread t at byte
-      // (((j + slot) mod PIECES) * NT + t) * 16 of slot `slot`, so that every wave instruction moves 1 KiB.
-      // The rotation by the slot index matters: the slots are 256 KiB apart, and workgroups that store
-      // (or load) piece j at the same moment at the same offset of their slots all meet on a few memory
-      // channels (measured: 20-25 us for the 256 KiB of a slot without it).
+      // (j * NT + t) * 16 of the piece's slot, so that every wave instruction moves 1 KiB.
       constexpr int PIECES = MB * NB * 4;  // 16-byte pieces per thread
       constexpr long long SLOT_BYTES = (long long)PIECES * NT * 16;
       if (item == ITEM_PART) {
@@ -937,7 +934,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           u32x4_t v;
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = __float_as_uint(acc_read(acc.v[mb][nb][4 * q + e]));
-          store16_system_of_valu_data(dst + (long long)((j + slot) % PIECES) * NT * 16, v);
+          store16_system_of_valu_data(dst + (long long)j * NT * 16, v);
           __builtin_amdgcn_sched_barrier(0);  // one piece at a time: the scheduler would read all 128 registers first
         }
         // Published like an aux tile: stores acknowledged by every wave, then one relaxed flag store.
@@ -1046,17 +1043,17 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           unsigned long long base = (unsigned long long)p.sk_partials + (unsigned long long)slot * SLOT_BYTES;
           asm volatile("" : "+s"(base));  // addresses are formed where they are used, not hoisted out of the tile loop
           const char* const src = (const char*)base + tid * 16;
-          auto load_batch = [&](u32x4_t (&dst)[BATCH], const char* src, int rot, int b) {  // rot: the slot's index
+          auto load_batch = [&](u32x4_t (&dst)[BATCH], const char* src, int b) {
 #pragma unroll
             for (int i = 0; i < BATCH; ++i)
-              dst[i] = __builtin_nontemporal_load((const u32x4_t*)(src + (long long)((b * BATCH + i + rot) % PIECES) * NT * 16));
+              dst[i] = __builtin_nontemporal_load((const u32x4_t*)(src + (long long)(b * BATCH + i) * NT * 16));
           };
           {  // the next batch is on its way while this one is staged
             u32x4_t buf[2][BATCH];
-            load_batch(buf[0], src, slot, 0);
+            load_batch(buf[0], src, 0);
 #pragma unroll
             for (int b = 0; b < NBATCH; ++b) {
-              if (b + 1 < NBATCH) load_batch(buf[(b + 1) & 1], src, slot, b + 1);
+              if (b + 1 < NBATCH) load_batch(buf[(b + 1) & 1], src, b + 1);
 #pragma unroll
               for (int i = 0; i < BATCH; ++i) {
                 float sum[4];
@@ -1431,27 +1428,17 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
   return launch_mfma_grid<CFG, false>(p, device, grid, stream);
 }
 
-// Tile shapes of the MFMA kernel.
-//   big     256x256, 8 waves, 4-slot ring: 128 accumulator registers per lane, the shape for large
-//           problems (half the operand bytes per flop of the 128x128 tiles).
-//   small   128x128, 4 waves, 128-byte K steps, 4-slot ring: for problems with too few big tiles.
-//   small2  128x128, 4 waves, 64-byte K steps, 4-slot ring of 64 KiB: two workgroups per CU.  For
-//           problems with more 128x128 tiles than CUs, where it keeps every tile resident at once
-//           instead of running a second, half-empty round (2048x2880x512: 39 -> 36 us); with fewer
-//           tiles the shorter K steps make it the slower of the two.
-//   skinny  64x128, 4 waves, 128-byte K steps, 3-slot ring of 72 KiB: two workgroups per CU.  Outputs of at
-//           most 64 rows that are too wide for the kernels below (fp16, two-shot, eight ranks, against the
-//           256x256 tile that the tile count alone would pick: 32x40960x2048 51 -> 38 us, 64x131072x2048
-//           150 -> 130 us), and outputs of 257-512 such tiles with a short K (at most 2048 bytes per row),
-//           where it is 8-13 % ahead of the 128x128 tiles (896x2880x512 18.6 -> 16.5 us, 1024x4096x512
-//           23.9 -> 21.9); at K = 1376 the two tie, at K = 4096 it is 10-20 % behind.  (With 256-byte steps
-//           and one workgroup per CU the same tile was 25-45 % slower on the wide outputs.)
-//   skinny64  64x64, 4 waves of one 32x32 block each, 128-byte K steps, 4-slot ring of 64 KiB (two
-//           workgroups per CU): outputs of at most two such tiles per CU, which wider tiles would spread
-//           over a part of the CUs.  (With 256-byte steps and three slots the same tile is 5-15 % slower:
-//           fp16, two-shot, eight ranks, 256x4096x512 12.2 against 11.6 us, 256x4096x4096 33.2 against 27.7.)
-// The small tiles keep as many bytes in flight as LDS allows; what pays is residency - every tile of the
-// output on a CU at the same time - before fat K steps.
+// Tile shapes of the MFMA kernel (run_fused picks one per launch).
+//   big       256x256, 8 waves, 64-byte K steps, 4-slot ring: half the operand bytes per flop of the
+//             128x128 tiles; from about half the CUs busy.
+//   small     128x128, 4 waves, 128-byte K steps, 4-slot ring: too few big tiles.
+//   small2    128x128, 4 waves, 64-byte K steps, 64 KiB ring, two workgroups per CU: more 128x128 tiles
+//             than CUs (every tile resident at once instead of a half-empty second round).
+//   skinny    64x128, 4 waves, 128-byte K steps, 72 KiB ring, two workgroups per CU: at most 64 rows, or at
+//             most two such tiles per CU with a short K.
+//   skinny64  64x64, 4 waves of one 32x32 block, 128-byte K steps, 64 KiB ring, two workgroups per CU: at
+//             most two such tiles per CU.
+// For the small tiles residency - every tile of the output on a CU at once - pays before fat K steps.
 enum { TILE_BIG = 0, TILE_SMALL = 1, TILE_SKINNY = 2, TILE_SMALL2 = 3, TILE_DECODE = 4, TILE_SKINNY64 = 5 };
 constexpr int tile_bk(int kind, int in) {  // K elements per step
   return (kind == TILE_BIG || kind == TILE_SMALL2 ? 64 : 128) / (in == IN_FP8 ? 1 : 2);

@@ -405,15 +405,9 @@ unsigned long long* g_stamps = nullptr;  // diagnostic build: where the kernels 
 long long g_stamp_rows = 0;              // ... and how many rows of 16 words the buffer holds
 #endif
 
-// Launches for the 32x32 kernel (decode_kernel.h): any output small enough that it has at most two 32x32
-// tiles per CU (two workgroups share a CU then) - decode-sized launches of up to 32 x 16384, and taller
-// ones of the same area.  Such outputs are a handful of
-// 128x128 tiles - 128 x 1024 is eight of them, on eight of 256 CUs - while the small tiles with K split
-// over the waves of a workgroup keep the whole chip busy (fp16, two-shot, eight ranks: 128x1024x4096 41 ->
-// 12 us, 64x2880x4096 35 -> 14 us, 256x2048x512 20 -> 9 us).
-// Beyond two tiles per CU the 64x64 tiled kernel is ahead at every K (fp16, 192x2880x4096: 25.0 against 29.4 us
-// for this kernel in a round of two and a round of one per CU; 640x1024x4096: 26.7 against 35.1; 32x32768x4096:
-// 51 against 66).
+// Launches for the 32x32 kernel (decode_kernel.h): outputs of at most two 32x32 tiles per CU.  Such an
+// output is a handful of 128x128 tiles on a handful of CUs, while 32x32 tiles with K split over the waves
+// of a workgroup keep the whole chip busy; beyond two tiles per CU the 64x64 tiled kernel is ahead.
 bool decode_sized(const FusedParams& p, int cu_count, int in_dtype) {
   if ((long long)cdiv(p.M, 32) * cdiv(p.N, 32) > 2ll * cu_count) return false;
   // ... and whose operands that kernel's 32-bit offsets reach (a tall A with long or padded rows does not
