@@ -332,14 +332,6 @@ __device__ __forceinline__ float acc_read(float a) {
   return v;
 }
 
-// a += x for a value that lives in an accumulation register, without the compiler moving the tile's
-// accumulators to VGPRs to do it.
-__device__ __forceinline__ float acc_add(float a, float x) {
-  float t;
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_add_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1" : "+a"(a), "=&v"(t) : "v"(x));
-  return a;
-}
-
 __device__ __forceinline__ unsigned lds_address(const void* p) {
   return (unsigned)(unsigned long long)(LDS_AS const char*)p;
 }
@@ -1157,9 +1149,9 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     if (flags) {
       // Publish: the aux tile was stored write-through at system scope; every wave waits until its
       // stores are acknowledged, the workgroup meets, and the threads that own flags raise them
-      // (no L2 write-back is needed any more).  Likewise the peers' flags are polled (system-scope
-      // acquire, which invalidates caches) by one set of threads for the whole workgroup; letting
-      // every wave poll and run ahead measured slower.
+      // (no L2 write-back is needed any more).  The peers' flags are polled by one set of threads for
+      // the whole workgroup (relaxed loads, one acquire when a flag is up); letting every wave poll
+      // and run ahead measured slower.
       // The peers' flags are looked at once while the own stores are still on their way: a thread that
       // found the flags it is responsible for up already - peers that finished first - has their round
       // trip hidden behind that wait and does not poll after the own flags are raised.  Every thread
