@@ -19,8 +19,8 @@ between flush and launch: the launch is queued while the flush kernel still runs
 holds the kernel and next to nothing of the host's launch path (5-8 us through Python, ctypes and the
 HIP runtime on an idle queue) and agrees with a profiler's kernel duration for the same command.
 `roofline` prices those launches (`priced_on`) against the roof that bounds the fused kernel (HBM for
-the slot-sum workloads, MFMA for the others); `frac_do_bench` is the same fraction priced on the literal
-do_bench launches, host path included; the back-to-back per-launch figures are carried as well;
+the slot-sum workloads, MFMA for the others); `frac_reference_protocol` (also at the top level of the line,
+next to `priced_on`) is the same fraction priced on the literal do_bench launches, host path included; the back-to-back per-launch figures are carried as well;
 `gemm_phase` repeats the measurement with the peers switched off (W = 1), which isolates the MFMA
 phase; `cpu_baseline` times torch's CPU matmul plus the slot reduction on the same workload.
 
@@ -570,6 +570,9 @@ def main():
         "config": wl.describe(args.world),
         "pct_of_mfma_peak": round(100 * tflops / PEAK[wl.dtype][0], 2) if wl.dtype in PEAK else None,
         "roofline": roofline,
+        # which launches roofline.frac is priced on, and the same fraction under the reference's literal protocol
+        "priced_on": priced_on,
+        "frac_reference_protocol": frac_reference,
     }
 
     if isinstance(wl, MatmulAllReduce) and not args.no_gemm_phase:
