@@ -62,6 +62,11 @@ struct FusedParams {
   long long spin_limit;
   int* status;
   int tiles_m, tiles_n, group_m, num_xcd;
+  // Tile order: 0 gives every XCD one contiguous span of the grouped order (tiles that share operand
+  // panels share an L2), 1 deals the grouped order out workgroup by workgroup (the chip works on one
+  // contiguous band of rows at a time; launches that stream the peers' tiles, see dispatch_mfma_in).
+  int interleave;
+  int group_m_spans;  // host only: the group height to use if the launch falls back to spans (split tiles)
   int row_offset;  // all-gather: first row of this rank's block in the gathered output
   // Heap bases as kernel arguments (slots 0..7), valid when hb_in_args is set: the host knew the contents
   // of the context tensor (iris_hip_register_context), which spares the kernels a dependent scalar load
@@ -620,6 +625,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
   // 2-3 us - passes under the epilogue.
   constexpr bool PREFETCH_NEXT = CFG::STAGE_SWIZZLED && !ONE_ROUND && !STREAMK;
   bool first_step_prefetched = false;
+  const int order_xcd = p.interleave ? 1 : p.num_xcd;  // see FusedParams::interleave
 
   for (int it = 0; ONE_ROUND ? it < 1 : true; ++it) {
     int tidx, k_begin = 0, k_end = nsteps, item = ITEM_WHOLE, partners = 0, slot = 0;
@@ -634,7 +640,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         slot += sk_slot0;
       }
     } else {
-      tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, p.num_xcd);
+      tidx = xcd_tile_index(blockIdx.x, gridDim.x, it, total_tiles, order_xcd);
       if (tidx < 0) break;
     }
     PHASE_STAMP(0);
@@ -957,7 +963,7 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
     }
 
     if constexpr (PREFETCH_NEXT) {
-      const int nidx = xcd_tile_index(blockIdx.x, gridDim.x, it + 1, total_tiles, p.num_xcd);
+      const int nidx = xcd_tile_index(blockIdx.x, gridDim.x, it + 1, total_tiles, order_xcd);
       if (nidx >= 0) {
         int ntm, ntn;
         grouped_tile(nidx, p.tiles_m, p.tiles_n, p.group_m, ntm, ntn);
@@ -1393,6 +1399,8 @@ int launch_mfma(const FusedParams& p, int device, int cu_count, hipStream_t stre
     FusedParams q = p;
     const int sk_grid = per_tile_launch ? 0 : split_tile_grid<CFG>(q, total, cu_count);
     if (sk_grid > 0) {
+      q.interleave = 0;  // the plan hands out the last round of every XCD's span
+      q.group_m = q.group_m_spans;
       constexpr long long slot_bytes = (long long)CFG::MB * CFG::NB * 4 * CFG::NT * 16;
       // No workspace (the stream is being captured before its first split launch, or the device has
       // used up its workspaces): hand the tiles out whole.
@@ -1472,10 +1480,18 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
   }
   p.tiles_m = cdiv(p.M, bm);
   p.tiles_n = cdiv(p.N, bn);
-  // Group height: tile-rows walked together so that an XCD's span of tiles is close to square.
+  // Group height: tile-rows walked together so that the tiles an XCD works on at one time - its whole
+  // span, or one round of it when the span is longer than its resident workgroups - are close to a
+  // square (fewest operand panels per L2).
   const int span = cdiv(p.tiles_m * p.tiles_n, p.num_xcd);
+  const int resident = (cu / p.num_xcd) * (kind == TILE_BIG || kind == TILE_SMALL ? 1 : 2);
+  const bool rounds = span > resident;
+  const int at_once = rounds ? resident : span;
   int g = 1;
-  while (g * g * 2 <= span && g * 2 <= p.tiles_m) g *= 2;
+  while (g * g * 2 <= at_once && g * 2 <= p.tiles_m) g *= 2;
+  // Two-shot launches of several rounds (one workgroup per tile, handed out in this order) do better with
+  // groups of at most four rows (eight ranks, fp16: 16384x3584x8192 1006 -> 977 us, 8192x8192x2752 441 -> 428).
+  if (rounds && p.sum_peers && p.world > 1 && p.epi == EPI_TWO_SHOT) g = g < 4 ? g : 4;
   // A reduce-scatter rank sums the slots only for its own band of rows.  With XCD spans that are
   // close to square that band falls to one or two XCDs, whose CUs then carry all the slow tiles;
   // taller groups spread it over more XCDs at the price of more operand panels per L2
@@ -1483,9 +1499,38 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
   // 16, 119 at 32; fetched by the L2s: 207, 290 and 443 MB).
   if (p.epi == EPI_REDUCE_SCATTER && !p.all_owners && p.sum_peers && p.world > 1)
     g = g * 2 < p.tiles_m ? g * 2 : p.tiles_m;
+  p.interleave = 0;
+  // The one-shot all-reduce with peers spends half its time streaming the peers' tiles, and that phase
+  // wants the workgroups that run together to read long pieces of the same rows (DRAM pages stay open):
+  // flat groups of two rows - more for narrow outputs, so that g x tiles_n stays near 32 (64 with two
+  // workgroups per CU) and an L2 still sees as few operand panels as with a square span.  When the
+  // launch fills the chip the grouped order is also dealt out workgroup by workgroup instead of in one
+  // span per XCD: XCD x then holds the tiles at positions x modulo the XCD count, 1/g of the rows and
+  // g/8 of the columns of one band of rows that the whole chip works on.  Measured, eight ranks, one box,
+  // square spans -> this rule: fp8 16384x8192x1024 568 -> 496 us (520 with flat spans), bf16
+  // 8192x4096x1376 216 -> 194, 4096x4096x1376 98.0 -> 96.8, 2048x8192x1376 108 -> 99, 2048x4096x1376
+  // (128x128 tiles) 64.6 -> 60.4, 256x4096x4096 (64x64 tiles, chip half full: spans) 39.3 -> 32.2.  Dealt
+  // out with one-row groups or spans of eight rows are the outliers (+9 % on 1536x6144x2048).  Two-shot
+  // launches lose 3-5 % when dealt out; launches without peers do not care.
+  if (p.epi == EPI_ONE_SHOT && p.sum_peers && p.world > 1) {
+    const int two_per_cu = !(kind == TILE_BIG || kind == TILE_SMALL);
+    g = 2;
+    while (g < 8 && g * 2 * p.tiles_n <= (two_per_cu ? 64 : 32)) g *= 2;
+    while (g > p.tiles_m && g > 1) g /= 2;
+    p.interleave = p.tiles_m * p.tiles_n >= resident * p.num_xcd;
+  }
+  p.group_m_spans = g;
+  static const int forced_order = [] {
+    const char* e = getenv("IRIS_HIP_TILE_ORDER");  // "spans" or "dealt": a tuning aid
+    return !e ? -1 : (e[0] == 'd' ? 1 : 0);
+  }();
+  if (forced_order >= 0) p.interleave = forced_order;
   // IRIS_HIP_GROUP_M overrides the group height (a tuning aid; results do not depend on the tile order).
   static const int forced_group_m = [] { const char* e = getenv("IRIS_HIP_GROUP_M"); return e ? atoi(e) : 0; }();
-  if (forced_group_m > 0) g = forced_group_m < p.tiles_m ? forced_group_m : p.tiles_m;
+  if (forced_group_m > 0) {
+    g = forced_group_m < p.tiles_m ? forced_group_m : p.tiles_m;
+    p.group_m_spans = g;
+  }
   p.group_m = g;
   static const char* names[3] = {"bf16", "f16", "fp8"};
   char name[96];
