@@ -1507,24 +1507,29 @@ int dispatch_mfma_in(FusedParams& p, int kind, bool bkc, int device, int cu, hip
     g = g * 2 < p.tiles_m ? g * 2 : p.tiles_m;
   p.interleave = 0;
   p.tile_rotate = 0;
-  // The one-shot all-reduce with peers spends half its time streaming the peers' tiles, and that phase
-  // wants the workgroups that run together to read long pieces of the same rows (DRAM pages stay open):
-  // flat groups of two rows - more for narrow outputs, so that g x tiles_n stays near 32 (64 with two
-  // workgroups per CU) and an L2 still sees as few operand panels as with a square span.  When the
-  // launch fills the chip the grouped order is also dealt out workgroup by workgroup instead of in one
-  // span per XCD: XCD x then holds the tiles at positions x modulo the XCD count, 1/g of the rows and
-  // g/8 of the columns of one band of rows that the whole chip works on.  Measured, eight ranks, one box,
-  // square spans -> this rule: fp8 16384x8192x1024 568 -> 496 us (520 with flat spans), bf16
-  // 8192x4096x1376 216 -> 194, 4096x4096x1376 98.0 -> 96.8, 2048x8192x1376 108 -> 99, 2048x4096x1376
-  // (128x128 tiles) 64.6 -> 60.4, 256x4096x4096 (64x64 tiles, chip half full: spans) 39.3 -> 32.2.  Dealt
-  // out with one-row groups or spans of eight rows are the outliers (+9 % on 1536x6144x2048).  Two-shot
-  // launches lose 3-5 % when dealt out; launches without peers do not care.
-  if (p.epi == EPI_ONE_SHOT && p.sum_peers && p.world > 1) {
+  // Launches whose epilogue streams whole tiles from or to every rank - the one-shot all-reduce with peers
+  // spends half its time reading the peers' tiles, matmul_all_gather and the atomic variant write every
+  // tile into all slots - want the workgroups that run together to touch long pieces of the same rows
+  // (DRAM pages stay open): flat groups of two rows - more for narrow outputs, so that g x tiles_n stays
+  // near 32 (64 with two workgroups per CU) and an L2 still sees as few operand panels as with a square
+  // span.  When the launch fills at least three quarters of the chip the grouped order is also dealt out
+  // workgroup by workgroup instead of in one span per XCD: XCD x then holds the tiles at positions x modulo
+  // the XCD count, 1/g of the rows and g/8 of the columns of one band of rows that the whole chip works on.
+  // Measured, eight ranks, one box, square spans -> this rule; one-shot: fp8 16384x8192x1024 568 -> 496 us
+  // (520 with flat spans), bf16 8192x4096x1376 216 -> 194, 4096x4096x1376 98.0 -> 96.8, 2048x8192x1376
+  // 108 -> 99, 2048x4096x1376 (128x128 tiles) 64.6 -> 60.4, 256x4096x4096 (64x64 tiles, chip half full:
+  // spans) 39.3 -> 32.2; atomic fp16 8192x4096x1376 566 -> 520; matmul_all_gather fp16 2048x3584x8192
+  // 175 -> 168, 512x4096x1376 22.9 -> 21.4.  Dealt out with one-row groups or spans of eight rows are the
+  // outliers (+9 % on 1536x6144x2048), and a chip that is little more than half full does better with spans
+  // (3072x3072x1024: 67.9 against 70.6).  Two-shot launches lose 3-5 % when dealt out; launches that
+  // neither read nor write other ranks' tiles do not care.
+  const bool streams_tiles = p.world > 1 && ((p.epi == EPI_ONE_SHOT && p.sum_peers) || p.epi == EPI_ALL_GATHER || p.epi == EPI_ATOMIC);
+  if (streams_tiles) {
     const int two_per_cu = !(kind == TILE_BIG || kind == TILE_SMALL);
     g = 2;
     while (g < 8 && g * 2 * p.tiles_n <= (two_per_cu ? 64 : 32)) g *= 2;
     while (g > p.tiles_m && g > 1) g /= 2;
-    p.interleave = p.tiles_m * p.tiles_n >= resident * p.num_xcd;
+    p.interleave = (long long)p.tiles_m * p.tiles_n * 4 >= (long long)resident * p.num_xcd * 3;
   }
   p.group_m_spans = g;
   // The reduce-scatter with peers is dealt out as well (its launches hand one workgroup per tile to the
