@@ -22,6 +22,11 @@ using namespace iris_layout;
 
 #define LDS_AS __attribute__((address_space(3)))
 
+// Stages of the slot-sum pipeline of the eight-wave tile (see reduce_chunks).
+#ifndef IRIS_HIP_EPILOGUE_DEPTH
+#define IRIS_HIP_EPILOGUE_DEPTH 2
+#endif
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -1206,90 +1211,121 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
         constexpr int NP = decltype(np_tag)::value;  // peers with cached bases; -1: any number
         constexpr bool RECT = decltype(rect_tag)::value;
         constexpr int NPV = NP > 0 ? NP : 1;
-        // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
-        // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
-        // at a time also with seven peers, and groups below the last row of the matrix are skipped.
-        constexpr int G0 = (NP >= 4 && NW == 8) ? 2 : 4;
-        constexpr int G = G0 < PASSES ? G0 : PASSES;
-        static_assert(PASSES % G == 0, "pass grouping");
         const int npasses = RECT ? cdiv((r1 - r0) * ncw, NT) : PASSES;
-        for (int pg = 0; pg < npasses; pg += G) {
-          if (!RECT && m0 + pg * RPP >= p.M) break;
-          bool active[G];
-          long long eoff[G];
-          int owner[G];
-          u32x4_t own[G], pv[G][NPV];
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            int gm, gc, lds_off;
-            if constexpr (RECT) {
-              const unsigned idx = (unsigned)((pg + g) * NT + tid);
-              const unsigned row = idx / (unsigned)ncw;
-              gm = r0 + (int)row;
-              gc = c0 + (int)(idx - row * (unsigned)ncw) * 8;
-              owner[g] = rect_owner;
-              active[g] = gm < r1;
-              lds_off = active[g] ? CFG::stage_offset(gm - m0, (gc - n0) * 2) : CFG::stage_offset(0, 0);
-            } else {
-              gm = m0 + (pg + g) * RPP + t_row;
-              gc = gn;
-              owner[g] = p.rank;
-              if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
-                const int t = (gm / p.flag_bm) * ftn + fcol;
-                owner[g] = owner_of(p.epi, t, ftotal, p.world, p.rank);
-              }
-              active[g] = gm < p.M && col_ok && (p.all_owners || owner[g] == p.rank);
-              lds_off = t_pass[(pg + g) & 1] + (pg + g) * RPP * CFG::TROW;
+        // One pass of the workgroup: the addresses of this thread's chunk, the peers' chunks requested, the
+        // own chunk read from LDS ...
+        struct Pass {
+          bool active;
+          long long eoff;
+          int owner;
+          u32x4_t own, pv[NPV];
+        };
+        auto issue = [&](int ps, Pass& st) {
+          int gm, gc, lds_off;
+          if constexpr (RECT) {
+            const unsigned idx = (unsigned)(ps * NT + tid);
+            const unsigned row = idx / (unsigned)ncw;
+            gm = r0 + (int)row;
+            gc = c0 + (int)(idx - row * (unsigned)ncw) * 8;
+            st.owner = rect_owner;
+            st.active = gm < r1;
+            lds_off = st.active ? CFG::stage_offset(gm - m0, (gc - n0) * 2) : CFG::stage_offset(0, 0);
+          } else {
+            gm = m0 + ps * RPP + t_row;
+            gc = gn;
+            st.owner = p.rank;
+            if (p.epi != EPI_ONE_SHOT) {  // one-shot reduces every tile: no owner arithmetic
+              const int t = (gm / p.flag_bm) * ftn + fcol;
+              st.owner = owner_of(p.epi, t, ftotal, p.world, p.rank);
             }
-            eoff[g] = active[g] ? ((long long)gm * p.s_cm + gc) * 2 : safe_off;
-            if constexpr (NP > 0) {
-#pragma unroll
-              for (int i = 0; i < NP; ++i) {
-                pv[g][i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + eoff[g]));
-              }
-            }
-            own[g] = *(const LDS_AS u32x4_t*)(LDS_AS char*)(smem + lds_off);
+            st.active = gm < p.M && col_ok && (p.all_owners || st.owner == p.rank);
+            lds_off = t_pass[ps & 1] + ps * RPP * CFG::TROW;
           }
+          st.eoff = st.active ? ((long long)gm * p.s_cm + gc) * 2 : safe_off;
+          if constexpr (NP > 0) {
 #pragma unroll
-          for (int g = 0; g < G; ++g) {
-            float sum[8];
+            for (int i = 0; i < NP; ++i) st.pv[i] = __builtin_nontemporal_load((const u32x4_t*)(pb[i] + st.eoff));
+          }
+          st.own = *(const LDS_AS u32x4_t*)(LDS_AS char*)(smem + lds_off);
+        };
+        // ... and its second half: the fp32 sum in ascending rank order from the own value, one cast, the stores.
+        auto finish = [&](const Pass& st) {
+          float sum[8];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sum[2 * e] = Out::to_float((unsigned short)(st.own[e] & 0xFFFF));
+            sum[2 * e + 1] = Out::to_float((unsigned short)(st.own[e] >> 16));
+          }
+          auto add_peer = [&](const u32x4_t& v) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              sum[2 * e] = Out::to_float((unsigned short)(own[g][e] & 0xFFFF));
-              sum[2 * e + 1] = Out::to_float((unsigned short)(own[g][e] >> 16));
+              sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
+              sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
             }
-            auto add_peer = [&](const u32x4_t& v) {
+            if (ref_chain) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                sum[2 * e] += Out::to_float((unsigned short)(v[e] & 0xFFFF));
-                sum[2 * e + 1] += Out::to_float((unsigned short)(v[e] >> 16));
-              }
-              if (ref_chain) {
+              for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
+            }
+          };
+          if constexpr (NP > 0) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sum[e] = Out::to_float(Out::from_float(sum[e]));
-              }
-            };
-            if constexpr (NP > 0) {
+            for (int i = 0; i < NP; ++i) add_peer(st.pv[i]);
+          } else if constexpr (NP < 0) {
+            for (int pr = 0; pr < p.world; ++pr)
+              if (pr != p.rank) add_peer(__builtin_nontemporal_load((const u32x4_t*)(in_slot(aux_own, pr) + st.eoff)));
+          }
+          u32x4_t res;
 #pragma unroll
-              for (int i = 0; i < NP; ++i) add_peer(pv[g][i]);
-            } else if constexpr (NP < 0) {
+          for (int e = 0; e < 4; ++e) res[e] = Out::pack(sum[2 * e], sum[2 * e + 1]);
+          if (st.active) {
+            if (p.epi == EPI_TWO_SHOT) {
+              __builtin_nontemporal_store(res, (u32x4_t*)(c_own + st.eoff));
               for (int pr = 0; pr < p.world; ++pr)
-                if (pr != p.rank) add_peer(__builtin_nontemporal_load((const u32x4_t*)(in_slot(aux_own, pr) + eoff[g])));
+                if (pr != p.rank) __builtin_nontemporal_store(res, (u32x4_t*)(in_slot(c_own, pr) + st.eoff));
+            } else {
+              const int dst = p.all_owners ? st.owner : p.rank;
+              __builtin_nontemporal_store(res, (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + st.eoff));
             }
-            u32x4_t res;
+          }
+        };
+        if constexpr (NW == 8 && NP >= 4 && ONE_ROUND) {
+          // Eight-wave tile with many peers, one tile per workgroup: the passes run as a pipeline of DEPTH
+          // stages - the loads of the next pass are on their way while one pass is summed and stored - so
+          // that the bytes a CU has in flight do not fall to zero between groups of passes (4096 x 4096 x 1376
+          // with seven peers: 92.9 -> 90.8 us against groups of two passes; three stages spill and gain
+          // nothing more).  Looping workgroups keep the groups: their launches run 1-7 % slower with the
+          // pipeline (fp8 16384 x 8192 x 1024: 494 -> 501 us with two stages, 527 with three) - a CU takes
+          // no more than about 39 GB/s of such loads however many are in flight, and the steadier stream
+          // of one workgroup only takes bandwidth from the others that are streaming at the time.
+          constexpr int DEPTH = IRIS_HIP_EPILOGUE_DEPTH;
+          const int last = RECT ? npasses : min(PASSES, cdiv(p.M - m0, RPP));  // passes below the last row of the matrix are skipped
+          Pass st[DEPTH];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              res[e] = Out::pack(sum[2 * e], sum[2 * e + 1]);
-            if (active[g]) {
-              if (p.epi == EPI_TWO_SHOT) {
-                __builtin_nontemporal_store(res, (u32x4_t*)(c_own + eoff[g]));
-                for (int pr = 0; pr < p.world; ++pr)
-                  if (pr != p.rank) __builtin_nontemporal_store(res, (u32x4_t*)(in_slot(c_own, pr) + eoff[g]));
-              } else {
-                const int dst = p.all_owners ? owner[g] : p.rank;
-                __builtin_nontemporal_store(res, (u32x4_t*)((dst == p.rank ? c_own : in_slot(c_own, dst)) + eoff[g]));
+          for (int d = 0; d < DEPTH; ++d)
+            if (d < last) issue(d, st[d]);
+          for (int ps = 0; ps < last; ps += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+              if (ps + d < last) {
+                finish(st[d]);
+                if (ps + d + DEPTH < last) issue(ps + d + DEPTH, st[d]);
               }
             }
+          }
+        } else {
+          // Passes whose loads are issued together.  Every group is one memory round trip (2 us on a
+          // launch of 10-20 us), so the four-wave tiles, which have the registers, take four passes
+          // at a time also with seven peers, and groups below the last row of the matrix are skipped.
+          constexpr int G0 = (NP >= 4 && NW == 8) ? 2 : 4;
+          constexpr int G = G0 < PASSES ? G0 : PASSES;
+          static_assert(PASSES % G == 0, "pass grouping");
+          for (int pg = 0; pg < npasses; pg += G) {
+            if (!RECT && m0 + pg * RPP >= p.M) break;
+            Pass st[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) issue(pg + g, st[g]);
+#pragma unroll
+            for (int g = 0; g < G; ++g) finish(st[g]);
           }
         }
       };
