@@ -1296,7 +1296,8 @@ __global__ void __launch_bounds__(CFG::NT, CFG::WAVES_PER_SIMD) fused_mfma_kerne
           // nothing more).  Looping workgroups keep the groups: their launches run 1-7 % slower with the
           // pipeline (fp8 16384 x 8192 x 1024: 494 -> 501 us with two stages, 527 with three) - a CU takes
           // no more than about 39 GB/s of such loads however many are in flight, and the steadier stream
-          // of one workgroup only takes bandwidth from the others that are streaming at the time.
+          // of one workgroup only takes bandwidth from the others that are streaming at the time.  The
+          // four-wave tiles gain nothing from a pipeline of four stages either (-2 to +3 % over ten shapes).
           constexpr int DEPTH = IRIS_HIP_EPILOGUE_DEPTH;
           const int last = RECT ? npasses : min(PASSES, cdiv(p.M - m0, RPP));  // passes below the last row of the matrix are skipped
           Pass st[DEPTH];
