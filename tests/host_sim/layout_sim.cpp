@@ -198,6 +198,40 @@ void check_tile_orders() {
       }
 }
 
+// The order launches that stream whole tiles use: the grouped order dealt out workgroup by workgroup
+// (xcd_tile_index with one "XCD"), optionally started `rotate` positions in (the reduce-scatter starts
+// at the rank's own band of rows).  Every tile exactly once; and with groups of g rows, XCD x (workgroup
+// index modulo 8) of a full first round meets 1/g of the round's tile rows and g/8 of its tile columns.
+void check_dealt_order() {
+  struct Case { int tm, tn, g, nwg, rotate; };
+  for (Case c : {Case{16, 16, 2, 256, 0}, Case{64, 32, 2, 256, 0}, Case{32, 16, 2, 256, 2 * 16 * 5}, Case{32, 16, 2, 512, 2 * 16 * 15},
+                 Case{7, 23, 2, 168, 46}, Case{32, 8, 4, 256, 0}}) {
+    const int total = c.tm * c.tn;
+    std::vector<int> count(total, 0);
+    for (int wg = 0; wg < c.nwg; ++wg)
+      for (int it = 0;; ++it) {
+        int idx = xcd_tile_index(wg, c.nwg, it, total, 1);
+        if (idx < 0) break;
+        idx += c.rotate;
+        if (idx >= total) idx -= total;
+        CHECK(idx >= 0 && idx < total, "dealt order out of range");
+        count[idx]++;
+      }
+    for (int t = 0; t < total; ++t) CHECK(count[t] == 1, "dealt order: tile %d taken %d times (tm=%d tn=%d)", t, count[t], c.tm, c.tn);
+  }
+  // 16 x 16 tiles, groups of two rows, 256 workgroups on 8 XCDs: each XCD sees 8 of the 16 tile rows and 4 of the 16 tile columns
+  for (int xcd = 0; xcd < 8; ++xcd) {
+    std::set<int> rows, cols;
+    for (int wg = xcd; wg < 256; wg += 8) {
+      int a, b;
+      grouped_tile(xcd_tile_index(wg, 256, 0, 256, 1), 16, 16, 2, a, b);
+      rows.insert(a);
+      cols.insert(b);
+    }
+    CHECK(rows.size() == 8 && cols.size() == 4, "dealt order: XCD %d meets %zu tile rows and %zu tile columns", xcd, rows.size(), cols.size());
+  }
+}
+
 // ---- flag tiles ----------------------------------------------------------------------------------------
 void check_flag_counts() {
   struct Case { int M, N, FM, FN, KM, KN; };
@@ -319,6 +353,7 @@ int main() {
   sim_col_operand<128, 1>(64);      // fp8 B tile 64 x 128
   check_acc_layout();
   check_tile_orders();
+  check_dealt_order();
   check_flag_counts();
   check_decode_offsets();
   check_split_plan();
